@@ -1,0 +1,142 @@
+/*
+ * moda_hip.h -- C ABI of libmoda_hip.so: fused sequence+depth attention
+ * (MoDA) for AMD MI355X (gfx950), forward and backward, plus the depth-KV
+ * cache reorganisation.
+ *
+ * Every pointer that names tensor data is a DEVICE pointer.  Strides are in
+ * elements; the innermost (head-dim) stride is always 1 and every row must be
+ * 16-byte aligned (base pointer and all strides multiples of 8 elements for
+ * 16-bit types, 4 for fp32).  All work is enqueued on the hipStream_t passed
+ * as `stream` (NULL = the legacy default stream); nothing synchronises the
+ * host.  The library keeps no mutable state except where a function says so.
+ * Every function returns 0 on success or a negative MODA_HIP_E* code; no
+ * function throws.
+ *
+ * Geometry (symbols as in the reference's docstrings):
+ *   folded layouts (modes CAUSAL, NONCAUSAL, CHUNK_VISIBLE, DEPTH_ONLY)
+ *     q, o, do, dq : [B, T*G, H, D]   query row r belongs to token r / G
+ *     k, v, dk, dv : [B, T,   H, D]
+ *     kd, vd, dkd, dvd : [B, T*L, H, D]   depth row t*L + l = slot l of token t
+ *     lse          : [B, T*G, H] fp32, base-2 log-sum-exp, contiguous
+ *   head-dim GQA layout (mode PLAIN_GQA, causal, no depth stream)
+ *     q, o, do, dq : [B, T, H*G, D]   query head hq reads kv head hq / G
+ *     lse          : [B, T, H*G]
+ */
+#ifndef MODA_HIP_H_
+#define MODA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MODA_HIP_VERSION 100
+
+enum moda_hip_dtype { MODA_HIP_BF16 = 0, MODA_HIP_FP16 = 1, MODA_HIP_FP32 = 2 };
+
+enum moda_hip_mode {
+  MODA_HIP_CAUSAL = 0,        /* moda_v14.py:45-378 with IS_CAUSAL=True            */
+  MODA_HIP_NONCAUSAL = 1,     /* moda_v14.py:259-300 (IS_CAUSAL=False)             */
+  MODA_HIP_CHUNK_VISIBLE = 2, /* moda_v16.py:39-352 (CHUNK_VISIBLE)                */
+  MODA_HIP_DEPTH_ONLY = 3,    /* fda_v12.py:44-253 (k, v are NULL)                 */
+  MODA_HIP_PLAIN_GQA = 4      /* fla/ops/attn/parallel.py:18-143 (kd, vd are NULL) */
+};
+
+enum moda_hip_error {
+  MODA_HIP_OK = 0,
+  MODA_HIP_EINVAL = -1,      /* bad descriptor field or NULL where data is required */
+  MODA_HIP_EUNSUPPORTED = -2,/* head dim / dtype combination without a kernel       */
+  MODA_HIP_EALIGN = -3,      /* pointer or stride not 16-byte aligned               */
+  MODA_HIP_EWORKSPACE = -4,  /* workspace too small                                 */
+  MODA_HIP_ELAUNCH = -5,     /* hipGetLastError() reported a launch failure         */
+  MODA_HIP_EDEVICE = -6      /* current device is not gfx950                        */
+};
+
+typedef struct moda_hip_strides {
+  int64_t b; /* batch stride   */
+  int64_t t; /* row stride     */
+  int64_t h; /* head stride    */
+} moda_hip_strides;
+
+typedef struct moda_hip_desc {
+  int32_t struct_size;  /* sizeof(moda_hip_desc), checked                         */
+  int32_t dtype;        /* moda_hip_dtype of q,k,v,kd,vd,o,do and all gradients    */
+  int32_t mode;         /* moda_hip_mode                                           */
+  int32_t reserved;
+  int64_t B;            /* batch                                                   */
+  int64_t T;            /* tokens (key rows)                                       */
+  int64_t H;            /* kv heads                                                */
+  int64_t G;            /* moda_group_num (folded) or query heads per kv head      */
+  int64_t D;            /* head dim of q/k and of v (must be equal)                */
+  int64_t L;            /* depth slots per token, 0 = no depth stream              */
+  int64_t chunk_tokens; /* CHUNK_VISIBLE: base tokens per chunk (C / G), else 0    */
+  float scale;          /* logits = scale * <q, key>                               */
+  float reserved_f;
+  moda_hip_strides q, k, v, kd, vd, o, d_o, dq, dk, dv, dkd, dvd;
+} moda_hip_desc;
+
+/*
+ * Forward.  Replaces parallel_moda_fwd + parallel_moda_fwd_kernel
+ * (moda_v14.py:381-522, 45-378), parallel_moda_chunk_visible_fwd
+ * (moda_v16.py:498-633), parallel_fda_fwd (fda_v12.py:261-400) and
+ * parallel_attn_fwd (fla/ops/attn/parallel.py:443-503).
+ * Writes o (dtype) and lse (fp32, base 2).  k, v NULL iff DEPTH_ONLY;
+ * kd, vd NULL iff L == 0.
+ */
+int moda_hip_fwd(const moda_hip_desc* desc, const void* q, const void* k, const void* v,
+                 const void* kd, const void* vd, void* o, float* lse, void* stream);
+
+/*
+ * Bytes of device workspace moda_hip_bwd needs (holds delta = rowsum(o * do),
+ * the quantity of moda_v14.py:525-539).  Returns 0 for an invalid descriptor.
+ */
+size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* desc);
+
+/*
+ * Backward.  Replaces parallel_moda_bwd and its kernels (moda_v14.py:1470-1842,
+ * 525-539, 542-871, 874-1248, 1251-1454), parallel_moda_chunk_visible_bwd
+ * (moda_v16.py:2099-2343), parallel_fda_bwd (fda_v12.py:881-1135) and
+ * parallel_attn_bwd (fla/ops/attn/parallel.py:522-629).
+ * Writes every element of dq, dk, dv, dkd, dvd (no pre-zeroing needed; nothing
+ * is accumulated with atomics, results are run-to-run identical).
+ * dk, dv NULL iff DEPTH_ONLY; dkd, dvd NULL iff L == 0.
+ */
+int moda_hip_bwd(const moda_hip_desc* desc, const void* q, const void* k, const void* v,
+                 const void* kd, const void* vd, const void* o, const float* lse, const void* d_o,
+                 void* dq, void* dk, void* dv, void* dkd, void* dvd,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Depth-KV reorganisation.  Replaces the caller-side
+ * torch.stack(dim=2).reshape(B, T*L, H, D).contiguous() of
+ * vision_tasks/deit/models.py:361-375 (one call per tensor, K or V).
+ * `layers` is a HOST array of n_layers device pointers, each a contiguous
+ * [B, T, H, D] tensor; they are written to slots [slot0, slot0 + n_layers) of
+ * the token-major cache [B, T*L_total, H, D].  With n_layers == 1 this is the
+ * in-place append of one layer's K (or V) into a preallocated cache.
+ */
+int moda_hip_depth_reorg_fwd(const void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total,
+                             int64_t B, int64_t T, int64_t H, int64_t D, int32_t dtype,
+                             void* cache, void* stream);
+
+/*
+ * Transpose of the above (the scatter autograd performs for the stack/reshape):
+ * splits d_cache [B, T*L_total, H, D] slots [slot0, slot0 + n_layers) into the
+ * per-layer gradients d_layers[i] ([B, T, H, D], contiguous, overwritten).
+ */
+int moda_hip_depth_reorg_bwd(const void* d_cache, int64_t n_layers, int64_t slot0, int64_t L_total,
+                             int64_t B, int64_t T, int64_t H, int64_t D, int32_t dtype,
+                             void* const* d_layers, void* stream);
+
+/* Human-readable text for an error code (static storage). */
+const char* moda_hip_strerror(int code);
+
+/* MODA_HIP_VERSION the library was built with. */
+int moda_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MODA_HIP_H_ */

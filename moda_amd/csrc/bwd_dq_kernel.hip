@@ -1,0 +1,222 @@
+// Backward, query side: delta = rowsum(o * do) (moda_v14.py:525-539) and the
+// dQ kernel (moda_v14.py:542-871, moda_v16.py:936-1220, fda_v12.py:432-638,
+// fla/ops/attn/parallel.py:165-296).
+//
+// Same decomposition as the forward kernel: a workgroup owns 128 query rows,
+// one row per lane pair, and streams 64-column K/V tiles (sequence keys, then
+// the rows' depth slots).  P^T is recomputed from the saved base-2 LSE,
+// dS^T = P^T * (dP^T - delta) is packed straight into the B operand of
+// dQ^T += K^T * dS^T, K^T coming from the LDS transpose read of the K tile.
+#include "kargs.h"
+#include "tile.h"
+
+namespace moda {
+
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void delta_kernel(const KArgs a) {
+  constexpr int TPR = HD / 8;         // threads per row
+  constexpr int RPB = 256 / TPR;      // rows per block
+  const int tid = threadIdx.x;
+  const int bh = blockIdx.y;
+  const int b = bh / a.Hq, hq = bh % a.Hq;
+  const int r = blockIdx.x * RPB + tid / TPR;
+  const int c = (tid % TPR) * 8;
+  float acc = 0.f;
+  if (r < a.Tq) {
+    const uint16_t* op = a.o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + c;
+    const uint16_t* dp = a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + c;
+    const typename T::vec8 ov = *reinterpret_cast<const typename T::vec8*>(op);
+    const typename T::vec8 dv = *reinterpret_cast<const typename T::vec8*>(dp);
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc += (float)ov[i] * (float)dv[i];
+  }
+#pragma unroll
+  for (int s = TPR / 2; s > 0; s >>= 1) acc += __shfl_xor(acc, s, 64);
+  if (r < a.Tq && (tid % TPR) == 0) a.delta[((int64_t)b * a.Hq + hq) * a.Tq + r] = acc;
+}
+
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void dq_kernel(const KArgs a) {
+  constexpr int BM = 128, BN = 64, KK = HD / 16, DB = HD / 32;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  uint16_t* smem = reinterpret_cast<uint16_t*>(smem_raw);
+  uint16_t* Ks[2] = {smem, smem + BN * HD};
+  uint16_t* Vs[2] = {smem + 2 * BN * HD, smem + 3 * BN * HD};
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
+  const int BH = a.B * a.Hq;
+  const int bh = blockIdx.x % BH;
+  const int qt = a.nqt - 1 - blockIdx.x / BH;
+  const int b = bh / a.Hq, hq = bh % a.Hq, hkv = hq / a.hdiv;
+  const int r = qt * BM + wave * 32 + n;
+  const bool valid = r < a.Tq;
+  const int t = r / a.Gf;
+
+  i32x4 Qr[KK], dOr[KK];
+  float lse = 0.f, delta = 0.f;
+  {
+    const uint16_t* qp = a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + 8 * g;
+    const uint16_t* dop = a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+      i32x4 z = {0, 0, 0, 0};
+      Qr[kk] = valid ? *reinterpret_cast<const i32x4*>(qp + 16 * kk) : z;
+      dOr[kk] = valid ? *reinterpret_cast<const i32x4*>(dop + 16 * kk) : z;
+    }
+    if (valid) {
+      lse = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq];
+      delta = a.delta[((int64_t)b * a.Hq + hq) * a.Tq + r];
+    }
+  }
+
+  int shi = 0, dlo = 0, dhi = 0;
+  if (valid) {
+    if (a.has_seq) shi = a.causal ? t + 1 : a.T;
+    if (a.L > 0) {
+      const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
+      dlo = lo_t * a.L;
+      dhi = (t + 1) * a.L;
+    }
+  }
+  const int r_first = qt * BM;
+  const int r_last = min(a.Tq, r_first + BM) - 1;
+  const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
+  int n_seq = 0;
+  if (a.has_seq) n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
+  int dep0 = 0, n_dep = 0;
+  if (a.L > 0) {
+    const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
+    dep0 = lo_t * a.L;
+    n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
+  }
+  const int ntiles = n_seq + n_dep;
+
+  const uint16_t* kb = a.has_seq ? a.k + b * a.sk.b + hkv * a.sk.h : nullptr;
+  const uint16_t* vb = a.has_seq ? a.v + b * a.sv.b + hkv * a.sv.h : nullptr;
+  const uint16_t* kdb = a.L > 0 ? a.kd + b * a.skd.b + hkv * a.skd.h : nullptr;
+  const uint16_t* vdb = a.L > 0 ? a.vd + b * a.svd.b + hkv * a.svd.h : nullptr;
+  const int TL = a.T * a.L;
+
+  TileLoader<HD, BN, 256> ldk, ldv;
+  auto issue = [&](int it) {
+    if (it < n_seq) {
+      ldk.load(kb, a.sk.t, it * BN, a.T, tid);
+      ldv.load(vb, a.sv.t, it * BN, a.T, tid);
+    } else {
+      const int c0 = dep0 + (it - n_seq) * BN;
+      ldk.load(kdb, a.skd.t, c0, TL, tid);
+      ldv.load(vdb, a.svd.t, c0, TL, tid);
+    }
+  };
+
+  f32x16 dq[DB];
+#pragma unroll
+  for (int d = 0; d < DB; d++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dq[d][i] = 0.f;
+  const float sc = a.scale * kLog2e;
+
+  if (ntiles > 0) {
+    issue(0);
+    ldk.store(Ks[0], tid);
+    ldv.store(Vs[0], tid);
+  }
+  __syncthreads();
+
+  for (int it = 0; it < ntiles; it++) {
+    const int cur = it & 1;
+    if (it + 1 < ntiles) issue(it + 1);
+
+    const bool dep = it >= n_seq;
+    const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
+    const int lo = dep ? dlo : 0;
+    const int hi = dep ? dhi : shi;
+    const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
+    if (__any(touches)) {
+      const bool full = (lo <= col0) && (hi >= col0 + BN);
+      const bool need_mask = !__all(full);
+      f32x16 s[2], dp[2];
+#pragma unroll
+      for (int bb = 0; bb < 2; bb++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          s[bb][i] = 0.f;
+          dp[bb][i] = 0.f;
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+          s[bb] = mfma32<T>(lds_row_operand<HD>(Ks[cur], 32 * bb, kk, lane), Qr[kk], s[bb]);
+          dp[bb] = mfma32<T>(lds_row_operand<HD>(Vs[cur], 32 * bb, kk, lane), dOr[kk], dp[bb]);
+        }
+      }
+#pragma unroll
+      for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          float p = fast_exp2(s[bb][i] * sc - lse);
+          if (need_mask) {
+            const int c = col0 + 32 * bb + acc_row(i, g);
+            p = (c >= lo && c < hi) ? p : 0.f;
+          }
+          s[bb][i] = p * (dp[bb][i] - delta);
+        }
+      i32x4 DS[4];
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) DS[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+#pragma unroll
+      for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+          dq[d] = mfma32<T>(lds_tr_operand<HD>(Ks[cur], 16 * ks, d, lane), DS[ks], dq[d]);
+    }
+
+    if (it + 1 < ntiles) {
+      ldk.store(Ks[cur ^ 1], tid);
+      ldv.store(Vs[cur ^ 1], tid);
+    }
+    __syncthreads();
+  }
+
+  if (valid) {
+    uint16_t* op = a.dq + b * a.sdq.b + hq * a.sdq.h + (int64_t)r * a.sdq.t;
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        i32x2 w;
+        w[0] = pack2<T>(dq[d][4 * i4 + 0] * a.scale, dq[d][4 * i4 + 1] * a.scale);
+        w[1] = pack2<T>(dq[d][4 * i4 + 2] * a.scale, dq[d][4 * i4 + 3] * a.scale);
+        *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
+      }
+  }
+}
+
+template <typename T, int HD>
+hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
+  constexpr size_t smem = 4 * 64 * HD * sizeof(uint16_t);
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<T, HD>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  if (a.Tq == 0 || a.B * a.Hq == 0) return hipSuccess;
+  constexpr int RPB = 256 / (HD / 8);
+  hipLaunchKernelGGL((delta_kernel<T, HD>), dim3((a.Tq + RPB - 1) / RPB, a.B * a.Hq), dim3(256), 0, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const int64_t nblk = (int64_t)a.nqt * a.B * a.Hq;
+  hipLaunchKernelGGL((dq_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), smem, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream) {
+  if (dtype == 0 && hd == 128) return launch_dq_t<BF16, 128>(a, stream);
+  if (dtype == 0 && hd == 64) return launch_dq_t<BF16, 64>(a, stream);
+  if (dtype == 1 && hd == 128) return launch_dq_t<FP16, 128>(a, stream);
+  if (dtype == 1 && hd == 64) return launch_dq_t<FP16, 64>(a, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace moda

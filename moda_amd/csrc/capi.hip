@@ -1,0 +1,267 @@
+// C ABI of libmoda_hip.so (see include/moda_hip.h): descriptor validation and
+// dispatch to the gfx950 kernels.  No tensor-library types cross this file.
+#include <hip/hip_runtime.h>
+#include <string.h>
+
+#include "../../include/moda_hip.h"
+#include "kargs.h"
+
+namespace moda {
+hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream);
+hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream);
+hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream);
+hipError_t launch_generic(const KArgs& a, int dtype, int D, int which, hipStream_t stream);
+hipError_t launch_reorg(void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t n_tokens,
+                        int64_t row_bytes, void* cache, bool to_cache, hipStream_t stream);
+}  // namespace moda
+
+using moda::KArgs;
+using moda::Str3;
+
+namespace {
+
+int elem_size(int dtype) { return dtype == MODA_HIP_FP32 ? 4 : 2; }
+
+Str3 cvt(const moda_hip_strides& s) { return Str3{s.b, s.t, s.h}; }
+
+bool aligned(const void* p, const moda_hip_strides& s, int esize) {
+  const int64_t m = 16 / esize;
+  return ((uintptr_t)p % 16 == 0) && (s.b % m == 0) && (s.t % m == 0) && (s.h % m == 0);
+}
+
+bool use_mfma(const moda_hip_desc* d) {
+  return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && (d->D == 64 || d->D == 128);
+}
+
+// Validates the descriptor and fills the geometry part of KArgs.
+int fill_geometry(const moda_hip_desc* d, KArgs& a) {
+  if (!d || d->struct_size != (int32_t)sizeof(moda_hip_desc)) return MODA_HIP_EINVAL;
+  if (d->dtype < MODA_HIP_BF16 || d->dtype > MODA_HIP_FP32) return MODA_HIP_EINVAL;
+  if (d->mode < MODA_HIP_CAUSAL || d->mode > MODA_HIP_PLAIN_GQA) return MODA_HIP_EINVAL;
+  if (d->B < 0 || d->T < 0 || d->H <= 0 || d->G <= 0 || d->D <= 0 || d->L < 0) return MODA_HIP_EINVAL;
+  if (d->D > 256 || d->D % 4 != 0) return MODA_HIP_EUNSUPPORTED;
+  if (d->mode == MODA_HIP_PLAIN_GQA && d->L != 0) return MODA_HIP_EINVAL;
+  if (d->mode == MODA_HIP_DEPTH_ONLY && d->L == 0) return MODA_HIP_EINVAL;
+  if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L > 0 && d->chunk_tokens <= 0) return MODA_HIP_EINVAL;
+  // 32-bit index space used for rows and flattened depth columns inside the kernels
+  if (d->T * d->G >= (1ll << 30) || d->T * (d->L > 0 ? d->L : 1) >= (1ll << 30) || d->B * d->H * d->G >= (1ll << 20))
+    return MODA_HIP_EUNSUPPORTED;
+  memset(&a, 0, sizeof(a));
+  const bool plain = d->mode == MODA_HIP_PLAIN_GQA;
+  a.B = (int)d->B;
+  a.T = (int)d->T;
+  a.Hkv = (int)d->H;
+  a.Tq = plain ? (int)d->T : (int)(d->T * d->G);
+  a.Gf = plain ? 1 : (int)d->G;
+  a.Hq = plain ? (int)(d->H * d->G) : (int)d->H;
+  a.hdiv = plain ? (int)d->G : 1;
+  a.L = (int)d->L;
+  a.Cb = d->mode == MODA_HIP_CHUNK_VISIBLE ? (int)(d->chunk_tokens > 0 ? d->chunk_tokens : 1) : 1;
+  a.has_seq = d->mode != MODA_HIP_DEPTH_ONLY;
+  a.causal = d->mode == MODA_HIP_CAUSAL || d->mode == MODA_HIP_CHUNK_VISIBLE || plain;
+  a.chunk = d->mode == MODA_HIP_CHUNK_VISIBLE;
+  a.nqt = (a.Tq + 127) / 128;
+  a.scale = d->scale;
+  return MODA_HIP_OK;
+}
+
+int check_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return MODA_HIP_EDEVICE;
+  static int cached_dev = -1;
+  static bool cached_ok = false;
+  if (dev != cached_dev) {
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, dev) != hipSuccess) return MODA_HIP_EDEVICE;
+    cached_ok = strncmp(p.gcnArchName, "gfx950", 6) == 0;
+    cached_dev = dev;
+  }
+  return cached_ok ? MODA_HIP_OK : MODA_HIP_EDEVICE;
+}
+
+#define MODA_REQ_PTR(p) \
+  if (!(p)) return MODA_HIP_EINVAL
+#define MODA_REQ_ALIGN(p, s) \
+  if (!aligned((p), (s), es)) return MODA_HIP_EALIGN
+
+}  // namespace
+
+extern "C" {
+
+int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
+                 const void* vd, void* o, float* lse, void* stream) {
+  KArgs a;
+  int rc = fill_geometry(d, a);
+  if (rc) return rc;
+  if ((int64_t)a.B * a.Tq * a.Hq == 0) return MODA_HIP_OK;
+  const int es = elem_size(d->dtype);
+  MODA_REQ_PTR(q);
+  MODA_REQ_PTR(o);
+  MODA_REQ_PTR(lse);
+  MODA_REQ_ALIGN(q, d->q);
+  MODA_REQ_ALIGN(o, d->o);
+  if (a.has_seq) {
+    MODA_REQ_PTR(k);
+    MODA_REQ_PTR(v);
+    MODA_REQ_ALIGN(k, d->k);
+    MODA_REQ_ALIGN(v, d->v);
+  }
+  if (a.L > 0) {
+    MODA_REQ_PTR(kd);
+    MODA_REQ_PTR(vd);
+    MODA_REQ_ALIGN(kd, d->kd);
+    MODA_REQ_ALIGN(vd, d->vd);
+  }
+  if ((rc = check_device())) return rc;
+  a.q = (const uint16_t*)q;
+  a.k = (const uint16_t*)k;
+  a.v = (const uint16_t*)v;
+  a.kd = (const uint16_t*)kd;
+  a.vd = (const uint16_t*)vd;
+  a.out_o = (uint16_t*)o;
+  a.lse = lse;
+  a.sq = cvt(d->q);
+  a.sk = cvt(d->k);
+  a.sv = cvt(d->v);
+  a.skd = cvt(d->kd);
+  a.svd = cvt(d->vd);
+  a.so = cvt(d->o);
+  hipError_t e = use_mfma(d) ? moda::launch_fwd(a, d->dtype, (int)d->D, (hipStream_t)stream)
+                             : moda::launch_generic(a, d->dtype, (int)d->D, 0, (hipStream_t)stream);
+  return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
+}
+
+size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* d) {
+  KArgs a;
+  if (fill_geometry(d, a)) return 0;
+  const size_t n = (size_t)a.B * a.Hq * a.Tq * sizeof(float);
+  return n ? n : sizeof(float);
+}
+
+int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
+                 const void* vd, const void* o, const float* lse, const void* d_o, void* dq, void* dk, void* dv,
+                 void* dkd, void* dvd, void* workspace, size_t workspace_bytes, void* stream) {
+  KArgs a;
+  int rc = fill_geometry(d, a);
+  if (rc) return rc;
+  const int es = elem_size(d->dtype);
+  const bool have_rows = (int64_t)a.B * a.Tq * a.Hq > 0;
+  if (have_rows) {
+    MODA_REQ_PTR(q);
+    MODA_REQ_PTR(o);
+    MODA_REQ_PTR(lse);
+    MODA_REQ_PTR(d_o);
+    MODA_REQ_PTR(dq);
+    MODA_REQ_ALIGN(q, d->q);
+    MODA_REQ_ALIGN(o, d->o);
+    MODA_REQ_ALIGN(d_o, d->d_o);
+    MODA_REQ_ALIGN(dq, d->dq);
+    if (a.has_seq) {
+      MODA_REQ_PTR(k);
+      MODA_REQ_PTR(v);
+      MODA_REQ_PTR(dk);
+      MODA_REQ_PTR(dv);
+      MODA_REQ_ALIGN(k, d->k);
+      MODA_REQ_ALIGN(v, d->v);
+      MODA_REQ_ALIGN(dk, d->dk);
+      MODA_REQ_ALIGN(dv, d->dv);
+    }
+    if (a.L > 0) {
+      MODA_REQ_PTR(kd);
+      MODA_REQ_PTR(vd);
+      MODA_REQ_PTR(dkd);
+      MODA_REQ_PTR(dvd);
+      MODA_REQ_ALIGN(kd, d->kd);
+      MODA_REQ_ALIGN(vd, d->vd);
+      MODA_REQ_ALIGN(dkd, d->dkd);
+      MODA_REQ_ALIGN(dvd, d->dvd);
+    }
+    if (!workspace || workspace_bytes < moda_hip_bwd_workspace_bytes(d)) return MODA_HIP_EWORKSPACE;
+  } else {
+    return MODA_HIP_OK;
+  }
+  if ((rc = check_device())) return rc;
+  a.q = (const uint16_t*)q;
+  a.k = (const uint16_t*)k;
+  a.v = (const uint16_t*)v;
+  a.kd = (const uint16_t*)kd;
+  a.vd = (const uint16_t*)vd;
+  a.o = (const uint16_t*)o;
+  a.d_o = (const uint16_t*)d_o;
+  a.lse = const_cast<float*>(lse);
+  a.delta = (float*)workspace;
+  a.dq = (uint16_t*)dq;
+  a.dk = (uint16_t*)dk;
+  a.dv = (uint16_t*)dv;
+  a.dkd = (uint16_t*)dkd;
+  a.dvd = (uint16_t*)dvd;
+  a.sq = cvt(d->q);
+  a.sk = cvt(d->k);
+  a.sv = cvt(d->v);
+  a.skd = cvt(d->kd);
+  a.svd = cvt(d->vd);
+  a.so = cvt(d->o);
+  a.sdo = cvt(d->d_o);
+  a.sdq = cvt(d->dq);
+  a.sdk = cvt(d->dk);
+  a.sdv = cvt(d->dv);
+  a.sdkd = cvt(d->dkd);
+  a.sdvd = cvt(d->dvd);
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  if (use_mfma(d)) {
+    e = moda::launch_dq(a, d->dtype, (int)d->D, s);
+    if (e == hipSuccess) e = moda::launch_dkv(a, d->dtype, (int)d->D, s);
+  } else {
+    e = moda::launch_generic(a, d->dtype, (int)d->D, 1, s);
+    if (e == hipSuccess) e = moda::launch_generic(a, d->dtype, (int)d->D, 2, s);
+  }
+  return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
+}
+
+int moda_hip_depth_reorg_fwd(const void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t B,
+                             int64_t T, int64_t H, int64_t D, int32_t dtype, void* cache, void* stream) {
+  if (n_layers < 0 || slot0 < 0 || slot0 + n_layers > L_total || B < 0 || T < 0 || H <= 0 || D <= 0)
+    return MODA_HIP_EINVAL;
+  if (dtype < MODA_HIP_BF16 || dtype > MODA_HIP_FP32) return MODA_HIP_EINVAL;
+  if (B * T == 0 || n_layers == 0) return MODA_HIP_OK;
+  if (!layers || !cache) return MODA_HIP_EINVAL;
+  for (int64_t i = 0; i < n_layers; i++)
+    if (!layers[i]) return MODA_HIP_EINVAL;
+  if (B * T >= (1ll << 31)) return MODA_HIP_EUNSUPPORTED;
+  hipError_t e = moda::launch_reorg(const_cast<void* const*>(layers), n_layers, slot0, L_total, B * T,
+                                    H * D * elem_size(dtype), cache, true, (hipStream_t)stream);
+  return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
+}
+
+int moda_hip_depth_reorg_bwd(const void* d_cache, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t B,
+                             int64_t T, int64_t H, int64_t D, int32_t dtype, void* const* d_layers, void* stream) {
+  if (n_layers < 0 || slot0 < 0 || slot0 + n_layers > L_total || B < 0 || T < 0 || H <= 0 || D <= 0)
+    return MODA_HIP_EINVAL;
+  if (dtype < MODA_HIP_BF16 || dtype > MODA_HIP_FP32) return MODA_HIP_EINVAL;
+  if (B * T == 0 || n_layers == 0) return MODA_HIP_OK;
+  if (!d_layers || !d_cache) return MODA_HIP_EINVAL;
+  for (int64_t i = 0; i < n_layers; i++)
+    if (!d_layers[i]) return MODA_HIP_EINVAL;
+  if (B * T >= (1ll << 31)) return MODA_HIP_EUNSUPPORTED;
+  hipError_t e = moda::launch_reorg(d_layers, n_layers, slot0, L_total, B * T, H * D * elem_size(dtype),
+                                    const_cast<void*>(d_cache), false, (hipStream_t)stream);
+  return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
+}
+
+const char* moda_hip_strerror(int code) {
+  switch (code) {
+    case MODA_HIP_OK: return "ok";
+    case MODA_HIP_EINVAL: return "invalid descriptor field or missing tensor pointer";
+    case MODA_HIP_EUNSUPPORTED: return "unsupported head dim / dtype / size";
+    case MODA_HIP_EALIGN: return "tensor pointer or stride is not 16-byte aligned";
+    case MODA_HIP_EWORKSPACE: return "workspace missing or too small";
+    case MODA_HIP_ELAUNCH: return "HIP kernel launch failed";
+    case MODA_HIP_EDEVICE: return "current device is not an MI355X-class (gfx950) GPU";
+    default: return "unknown error";
+  }
+}
+
+int moda_hip_version(void) { return MODA_HIP_VERSION; }
+
+}  // extern "C"

@@ -1,0 +1,176 @@
+// Device-side building blocks shared by the gfx950 attention kernels:
+// 16-bit element types, MFMA 32x32x16 wrappers, the swizzled LDS tile layout
+// and its two read patterns (row operand, transposed operand).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace moda {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+struct BF16 {
+  typedef bf16x8 vec8;
+  typedef bf16x4 vec4;
+  typedef __bf16 elem;
+};
+struct FP16 {
+  typedef f16x8 vec8;
+  typedef f16x4 vec4;
+  typedef _Float16 elem;
+};
+
+#define MODA_LDS __attribute__((address_space(3)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+// D(32x32) += A(32x16) * B(16x32).  Operand layout per lane l (n = l & 31,
+// g = l >> 5): A holds row n, k = 8g..8g+7; B holds column n, k = 8g..8g+7;
+// the accumulator holds column n, rows (i/4)*8 + 4g + (i%4) for i = 0..15.
+template <typename T>
+__device__ __forceinline__ f32x16 mfma32(i32x4 a, i32x4 b, f32x16 c);
+template <>
+__device__ __forceinline__ f32x16 mfma32<BF16>(i32x4 a, i32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16 mfma32<FP16>(i32x4 a, i32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
+                                                0);
+}
+
+// Row index inside a 32-row accumulator block that register i of lane-half g holds.
+__device__ __forceinline__ constexpr int acc_row(int i, int g) { return (i >> 2) * 8 + g * 4 + (i & 3); }
+
+// fp32 -> 16-bit packs (round to nearest even).
+template <typename T>
+__device__ __forceinline__ int pack2(float a, float b);
+template <>
+__device__ __forceinline__ int pack2<BF16>(float a, float b) {
+  bf16x2 v;
+  v[0] = (__bf16)a;
+  v[1] = (__bf16)b;
+  return __builtin_bit_cast(int, v);
+}
+template <>
+__device__ __forceinline__ int pack2<FP16>(float a, float b) {
+  f16x2 v;
+  v[0] = (_Float16)a;
+  v[1] = (_Float16)b;
+  return __builtin_bit_cast(int, v);
+}
+
+// Eight consecutive accumulator registers -> one MFMA B operand (k slots 0..7).
+template <typename T>
+__device__ __forceinline__ i32x4 pack8(const f32x16& x, int first) {
+  i32x4 r;
+  r[0] = pack2<T>(x[first + 0], x[first + 1]);
+  r[1] = pack2<T>(x[first + 2], x[first + 3]);
+  r[2] = pack2<T>(x[first + 4], x[first + 5]);
+  r[3] = pack2<T>(x[first + 6], x[first + 7]);
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ float to_float(typename T::elem x) {
+  return (float)x;
+}
+
+// ---------------------------------------------------------------------------
+// LDS tile: ROWS x HD 16-bit elements, row-major, 16-byte chunks XOR-swizzled
+// so that (a) 16 consecutive rows at one logical chunk and (b) 4 consecutive
+// rows x 4 adjacent chunks both spread over all banks.
+// ---------------------------------------------------------------------------
+template <int HD>
+struct Tile {
+  static constexpr int CH = HD / 8;  // 16-byte chunks per row
+  __device__ __forceinline__ static int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (CH - 1); }
+  // element offset of logical (row, chunk)
+  __device__ __forceinline__ static int off(int row, int chunk) { return row * HD + ((chunk ^ swz(row)) << 3); }
+};
+
+// Row operand: lane (n, g) gets elements [16*kk + 8g, +8) of row (row0 + n).
+// Serves as MFMA A (M = tile rows) or B (N = tile rows) with K = head dim.
+template <int HD>
+__device__ __forceinline__ i32x4 lds_row_operand(const uint16_t* tile, int row0, int kk, int lane) {
+  const int n = lane & 31, g = lane >> 5;
+  const uint16_t* p = tile + Tile<HD>::off(row0 + n, 2 * kk + g);
+  return *reinterpret_cast<const i32x4*>(p);
+}
+
+// Transposed operand: lane (n, g) gets, for head-dim column d = 32*dblk + n,
+// tile rows rb + 4g + {0,1,2,3} (k slots 0..3) and rb + 8 + 4g + {0,1,2,3}
+// (k slots 4..7) -- exactly the rows that accumulator registers 8s..8s+7 of a
+// 32-row block hold, so a packed accumulator can be the other operand.
+// Uses the gfx950 LDS transpose read: within each 16-lane group, source lane
+// r supplies the address of 4 consecutive elements; result lane i receives
+// element (i & 3) of source lanes 4j + (i >> 2), j = 0..3.
+template <int HD>
+__device__ __forceinline__ i32x4 lds_tr_operand(const uint16_t* tile, int rb, int dblk, int lane) {
+  const int g = lane >> 5;
+  const int r16 = lane & 15;
+  const int row = rb + 4 * g + (r16 >> 2);
+  const int dcol = 32 * dblk + ((lane >> 4) & 1) * 16 + (r16 & 3) * 4;
+  const uint16_t* p0 = tile + Tile<HD>::off(row, dcol >> 3) + (dcol & 7);
+  const uint16_t* p1 = tile + Tile<HD>::off(row + 8, dcol >> 3) + (dcol & 7);
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(p0));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(p1));
+  i32x2 l2 = __builtin_bit_cast(i32x2, lo);
+  i32x2 h2 = __builtin_bit_cast(i32x2, hi);
+  i32x4 r;
+  r[0] = l2[0];
+  r[1] = l2[1];
+  r[2] = h2[0];
+  r[3] = h2[1];
+  return r;
+}
+
+// Cooperative global -> register -> LDS staging of a ROWS x HD tile by NT threads.
+// Rows outside [0, nrows) relative to `base` read as zero.
+template <int HD, int ROWS, int NT>
+struct TileLoader {
+  static constexpr int CH = HD / 8;
+  static constexpr int N = (ROWS * CH) / NT;  // 16-byte chunks per thread
+  static_assert((ROWS * CH) % NT == 0, "tile must divide evenly");
+  i32x4 r[N];
+
+  // src points at row 0 of the (batch, head) slice; rows outside [0, row_end) are zero-filled
+  __device__ __forceinline__ void load(const uint16_t* src, int64_t row_stride, int64_t row0, int64_t row_end,
+                                       int tid) {
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      const int id = tid + i * NT;
+      const int row = id / CH, ch = id % CH;
+      const int64_t gr = row0 + row;
+      i32x4 v = {0, 0, 0, 0};
+      if (gr >= 0 && gr < row_end) v = *reinterpret_cast<const i32x4*>(src + gr * row_stride + ch * 8);
+      r[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(uint16_t* tile, int tid) const {
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      const int id = tid + i * NT;
+      const int row = id / CH, ch = id % CH;
+      *reinterpret_cast<i32x4*>(tile + Tile<HD>::off(row, ch)) = r[i];
+    }
+  }
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+
+}  // namespace moda

@@ -1,0 +1,556 @@
+"""Host side of the fused sequence+depth attention operators.
+
+Mirrors the reference's Python operator interface -- same function names,
+argument meaning, assertions and return conventions -- on top of the C ABI of
+``libmoda_hip.so``:
+
+  * ``parallel_moda`` / ``parallel_moda_fwd`` / ``parallel_moda_bwd``
+    (libs/moda_triton/fla/ops/moda/moda_v14.py:2792-2893, 381-522, 1470-1842)
+  * ``parallel_moda_chunk_visible`` / ``_fwd`` / ``_bwd``
+    (moda_v16.py:3614-3651, 498-633, 2099-2343)
+  * ``parallel_fda`` / ``_fwd`` / ``_bwd`` (fda_v12.py:1346-1449, 261-400, 881-1135)
+  * ``parallel_attn`` (fla/ops/attn/parallel.py:678-730), the plain causal comparator.
+
+Tensors stay torch tensors; torch is used for allocation, streams and autograd
+only.  Every compute step is a HIP kernel of the shared library.
+"""
+from __future__ import annotations
+
+import ctypes
+import warnings
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import Desc, Strides
+
+_DTYPES = {torch.bfloat16: _lib.BF16, torch.float16: _lib.FP16, torch.float32: _lib.FP32}
+
+# Query rows per chunk of the chunk-visible variant when the caller does not
+# say: the value the reference hard-wires in its launchers (moda_v16.py:581-585).
+DEFAULT_CHUNK_ROWS = 64
+
+
+def _ptr(x: Optional[torch.Tensor]):
+    return ctypes.c_void_p(x.data_ptr()) if x is not None else ctypes.c_void_p(0)
+
+
+def _stream(x: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+
+
+def _usable(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """Return ``x`` if the kernels can read it in place (unit inner stride, 16-byte
+    aligned rows), else a contiguous copy -- the reference's ``@contiguous``
+    (fla/utils.py:130-164) made a copy of every non-contiguous input."""
+    if x is None:
+        return None
+    m = 16 // x.element_size()
+    ok = (
+        x.dim() == 4
+        and (x.stride(3) == 1 or x.shape[3] == 1)
+        and all(x.stride(i) % m == 0 for i in range(3))
+        and x.data_ptr() % 16 == 0
+        and all(x.stride(i) >= 0 for i in range(3))
+    )
+    return x if ok else x.contiguous()
+
+
+def _strides(x: Optional[torch.Tensor]) -> Strides:
+    if x is None:
+        return Strides(0, 0, 0)
+    return Strides(x.stride(0), x.stride(1), x.stride(2))
+
+
+def _check_device(x: torch.Tensor):
+    if not x.is_cuda:
+        raise RuntimeError(
+            "moda_amd operators run only on an MI355X (gfx950) device tensor; there is no CPU path"
+        )
+
+
+def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=None, dk=None, dv=None, dkd=None,
+          dvd=None) -> Desc:
+    d = Desc()
+    d.struct_size = ctypes.sizeof(Desc)
+    if q.dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {q.dtype}; expected bf16, fp16 or fp32")
+    d.dtype = _DTYPES[q.dtype]
+    d.mode = mode
+    src = kd if mode == _lib.DEPTH_ONLY else k
+    d.B = q.shape[0]
+    d.H = src.shape[2]
+    d.G = G
+    d.D = q.shape[3]
+    d.L = L
+    if mode == _lib.DEPTH_ONLY:
+        d.T = q.shape[1] // G
+    else:
+        d.T = k.shape[1]
+    d.chunk_tokens = chunk_tokens
+    d.scale = float(scale)
+    d.q, d.k, d.v, d.kd, d.vd = _strides(q), _strides(k), _strides(v), _strides(kd), _strides(vd)
+    d.o, d.d_o = _strides(o), _strides(do)
+    d.dq, d.dk, d.dv, d.dkd, d.dvd = _strides(dq), _strides(dk), _strides(dv), _strides(dkd), _strides(dvd)
+    return d
+
+
+def _same_dtype(*xs):
+    dt = None
+    for x in xs:
+        if x is None:
+            continue
+        if dt is None:
+            dt = x.dtype
+        elif x.dtype != dt:
+            raise TypeError(f"all tensors must share one dtype, got {dt} and {x.dtype}")
+
+
+def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0):
+    """Launch the forward kernels. Returns (o, lse)."""
+    _check_device(q)
+    _same_dtype(q, k, v, kd, vd)
+    q, k, v, kd, vd = map(_usable, (q, k, v, kd, vd))
+    src = kd if mode == _lib.DEPTH_ONLY else k
+    T = q.shape[1] // G if mode == _lib.DEPTH_ONLY else k.shape[1]
+    L = (kd.shape[1] // T) if (kd is not None and T > 0) else 0
+    if kd is not None and T == 0:
+        L = 0
+    val = vd if mode == _lib.DEPTH_ONLY else v
+    if val.shape[-1] != q.shape[-1]:
+        raise NotImplementedError("value head dim must equal key head dim")
+    o = torch.empty(q.shape[0], q.shape[1], q.shape[2], val.shape[-1], dtype=val.dtype, device=q.device)
+    lse = torch.empty(q.shape[0], q.shape[1], q.shape[2], dtype=torch.float32, device=q.device)
+    if L == 0:
+        kd = vd = None
+    d = _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=o)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().moda_hip_fwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kd), _ptr(vd), _ptr(o),
+                                      _ptr(lse), _stream(q))
+    _lib.check(rc, "moda_hip_fwd")
+    return o, lse
+
+
+def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0):
+    """Launch the backward kernels. Returns (dq, dk, dv, dkd, dvd)."""
+    _check_device(q)
+    _same_dtype(q, k, v, kd, vd, o, do)
+    q, k, v, kd, vd, o, do = map(_usable, (q, k, v, kd, vd, o, do))
+    lse = lse.contiguous()
+    T = q.shape[1] // G if mode == _lib.DEPTH_ONLY else k.shape[1]
+    L = (kd.shape[1] // T) if (kd is not None and T > 0) else 0
+    dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    dk = torch.empty(k.shape, dtype=k.dtype, device=q.device) if k is not None else None
+    dv = torch.empty(v.shape, dtype=v.dtype, device=q.device) if v is not None else None
+    dkd = torch.empty(kd.shape, dtype=kd.dtype, device=q.device) if kd is not None else None
+    dvd = torch.empty(vd.shape, dtype=vd.dtype, device=q.device) if vd is not None else None
+    kd_a, vd_a, dkd_a, dvd_a = (kd, vd, dkd, dvd) if L > 0 else (None, None, None, None)
+    d = _desc(mode, q, k, v, kd_a, vd_a, G, L, chunk_tokens, scale, o=o, do=do, dq=dq, dk=dk, dv=dv, dkd=dkd_a,
+              dvd=dvd_a)
+    lib = _lib.load()
+    nbytes = lib.moda_hip_bwd_workspace_bytes(ctypes.byref(d))
+    ws = torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.moda_hip_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kd_a), _ptr(vd_a), _ptr(o), _ptr(lse),
+                              _ptr(do), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dkd_a), _ptr(dvd_a), _ptr(ws),
+                              ctypes.c_size_t(ws.numel()), _stream(q))
+    _lib.check(rc, "moda_hip_bwd")
+    return dq, dk, dv, dkd, dvd
+
+
+# ---------------------------------------------------------------------------
+# MoDA (causal / non-causal)  -- moda_v14.py
+# ---------------------------------------------------------------------------
+def _assert_group_tile(moda_group_num: int, rows: int = 128):
+    assert (
+        rows % moda_group_num == 0
+    ), "To keep depth alignment consistent with backward, BT % moda_group_num must be 0"
+
+
+def parallel_moda_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, cached_v=None, moda_group_num=1,
+                      is_causal=True, customized_BT=None, customized_BS=None, customized_BK=None, customized_BV=None,
+                      customized_num_warps=None):
+    """moda_v14.py:381-522.  Returns ``(o, lse)``; tile-size knobs are accepted and ignored."""
+    assert g_cumsum is None, "g_cumsum is not supported in this version"
+    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    assert q.shape[2] == k.shape[2], (
+        "Implicit head-dimension GQA is not allowed. "
+        "Please fold grouping only into `moda_group_num`: "
+        "use q.shape[2] == k.shape[2] and set T_q = T_kv * moda_group_num."
+    )
+    _assert_group_tile(moda_group_num)
+    mode = _lib.CAUSAL if is_causal else _lib.NONCAUSAL
+    return _raw_fwd(mode, q, k, v, cached_k, cached_v, scale, moda_group_num)
+
+
+def parallel_moda_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None, cached_k=None,
+                      cached_v=None, moda_group_num=1, is_causal=True, customized_BT=None, customized_BS=None,
+                      customized_BK=None, customized_BV=None, customized_num_warps=None, group_bs=None,
+                      group_warps=None, depth_bs=None, depth_warps=None):
+    """moda_v14.py:1470-1842.  Returns ``(dq, dk, dv, dg_cumsum=None, d_cached_k, d_cached_v)``."""
+    assert g_cumsum is None, "g_cumsum is not supported in this version"
+    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    assert q.shape[2] == k.shape[2], (
+        "Implicit head-dimension GQA is not allowed. "
+        "Please fold grouping only into `moda_group_num`: "
+        "use q.shape[2] == k.shape[2] and set T_q = T_kv * moda_group_num."
+    )
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    _assert_group_tile(moda_group_num)
+    mode = _lib.CAUSAL if is_causal else _lib.NONCAUSAL
+    dq, dk, dv, dkd, dvd = _raw_bwd(mode, q, k, v, cached_k, cached_v, o, lse, do, scale, moda_group_num)
+    return dq, dk, dv, None, dkd, dvd
+
+
+def _autograd_forward(ctx, fwd_impl, q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, **kw):
+    assert g is None, "g is not supported in this version"
+    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    has_depth = cached_k is not None and cached_v is not None
+    if not has_depth:
+        cached_k = cached_v = None
+    o, lse = fwd_impl(q=q, k=k, v=v, g_cumsum=None, scale=scale, cu_seqlens=None, cached_k=cached_k,
+                      cached_v=cached_v, moda_group_num=moda_group_num, **kw)
+    ctx.save_for_backward(q, k, v, o, lse, *([cached_k, cached_v] if has_depth else []))
+    ctx.has_depth = has_depth
+    ctx.scale = scale
+    ctx.moda_group_num = moda_group_num
+    ctx.kw = kw
+    return o.to(q.dtype), lse
+
+
+def _autograd_backward(ctx, bwd_impl, do):
+    if ctx.has_depth:
+        q, k, v, o, lse, cached_k, cached_v = ctx.saved_tensors
+    else:
+        q, k, v, o, lse = ctx.saved_tensors
+        cached_k = cached_v = None
+    dq, dk, dv, _, dkd, dvd = bwd_impl(q=q, k=k, v=v, o=o, g_cumsum=None, lse=lse, do=do.to(o.dtype), scale=ctx.scale,
+                                       cu_seqlens=None, cached_k=cached_k, cached_v=cached_v,
+                                       moda_group_num=ctx.moda_group_num, **ctx.kw)
+    if not ctx.has_depth:
+        dkd = dvd = None
+    return dq.to(q), dk.to(k), dv.to(v), dkd, dvd
+
+
+class ParallelMixtureOfDepthAttentionFunction(torch.autograd.Function):
+    """moda_v14.py:2649-2789: 14 inputs, 14 gradients, gradient into ``lse`` ignored."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, q, k, v, g, scale, cu_seqlens, cached_k=None, cached_v=None, moda_group_num=1, is_causal=True,
+                group_bs=None, group_warps=None, depth_bs=None, depth_warps=None):
+        o, lse = _autograd_forward(ctx, parallel_moda_fwd, q, k, v, g, scale, cu_seqlens, cached_k, cached_v,
+                                   moda_group_num, is_causal=is_causal)
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, do, dlse_unused):
+        dq, dk, dv, dkd, dvd = _autograd_backward(ctx, parallel_moda_bwd, do)
+        return dq, dk, dv, None, None, None, dkd, dvd, None, None, None, None, None, None
+
+
+def _prepare_inputs(api_name, q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first,
+                    return_depth_grads, warn_shape):
+    """Shared argument contract of parallel_moda (moda_v14.py:2817-2871) and
+    parallel_moda_chunk_visible (moda_v16.py:3496-3565)."""
+    if head_first:
+        q = q.transpose(1, 2)
+        k = k.transpose(1, 2)
+        v = v.transpose(1, 2)
+        if g is not None:
+            g = g.transpose(1, 2)
+        if cached_k is not None and cached_v is not None:
+            cached_k = cached_k.transpose(1, 2)
+            cached_v = cached_v.transpose(1, 2)
+    elif warn_shape and q.shape[1] < q.shape[2]:
+        warnings.warn(
+            f"[{api_name}] detected seq_len({q.shape[1]}) < num_heads({q.shape[2]}). "
+            "input may be in head_first format while head_first=True is not set."
+        )
+    B, T_q, HQ, Kdim = q.shape
+    T_kv = k.shape[1]
+    H = k.shape[2]
+    assert HQ == H, (
+        "Implicit head-dimension GQA is not allowed. "
+        "Please fold grouping only into `moda_group_num`: "
+        "use q.shape[2] == k.shape[2] and set T_q = T_kv * moda_group_num."
+    )
+    if scale is None:
+        scale = Kdim ** -0.5
+    if moda_group_num > 1:
+        assert T_q == T_kv * moda_group_num, "When moda_group_num > 1, T_q must equal T_kv * moda_group_num"
+    else:
+        assert T_q == T_kv, "When moda_group_num=1, T_q must equal T_kv"
+    if cached_k is not None and cached_v is not None:
+        assert cached_k.shape[0] == B and cached_v.shape[0] == B
+        assert cached_k.shape[2] == H and cached_v.shape[2] == H, "cached_k/v head count mismatch"
+        assert cached_k.shape[1] % T_kv == 0, "cached_k time dimension must be T_kv * L"
+        L = cached_k.shape[1] // T_kv
+        assert cached_v.shape[1] == T_kv * L, "cached_v shape mismatch"
+        if (cached_k.requires_grad or cached_v.requires_grad) and not return_depth_grads:
+            warnings.warn(
+                "cached_k/v requires gradients, but return_depth_grads=False. "
+                "Gradients are still computed and returned."
+            )
+    if g is not None:
+        assert g.shape[:3] == (B, T_q, HQ), "g must be [B,T_q,HQ]"
+    return q, k, v, g, cached_k, cached_v, scale
+
+
+def parallel_moda(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_seqlens=None, moda_group_num=1,
+                  is_causal=True, head_first=False, need_lse=False, return_depth_grads=True, warn_shape=True,
+                  customized_BT=None, customized_BS=None, customized_BT_backward=None, customized_BS_backward=None,
+                  group_bs=None, group_warps=None, depth_bs=None, depth_warps=None):
+    """Fused sequence+depth attention; signature of moda_v14.py:2792-2815.
+
+    q ``[B, T*G, H, D]``; k, v ``[B, T, H, D]``; cached_k/v ``[B, T*L, H, D]`` or
+    None.  Returns ``o`` (q.dtype) or ``(o, lse)`` with ``lse`` fp32 in base-2
+    units.  The ``customized_*``, ``group_*`` and ``depth_*`` knobs tune the
+    reference's Triton launches and have no meaning here; they are accepted and
+    ignored.
+    """
+    q, k, v, g, cached_k, cached_v, scale = _prepare_inputs(
+        "parallel_moda", q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first, return_depth_grads,
+        warn_shape)
+    o, lse = ParallelMixtureOfDepthAttentionFunction.apply(
+        q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, is_causal, group_bs, group_warps, depth_bs,
+        depth_warps)
+    return (o, lse) if need_lse else o
+
+
+# ---------------------------------------------------------------------------
+# chunk-visible MoDA -- moda_v16.py
+# ---------------------------------------------------------------------------
+def _chunk_tokens(moda_group_num: int, customized_BT: Optional[int]) -> int:
+    rows = customized_BT if customized_BT is not None else DEFAULT_CHUNK_ROWS
+    assert (
+        rows % moda_group_num == 0
+    ), "BT must be divisible by moda_group_num to keep chunk-visible base_t aligned"
+    return rows // moda_group_num
+
+
+def parallel_moda_chunk_visible_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, cached_v=None,
+                                    moda_group_num=1, customized_BT=None, customized_BS=None, customized_BK=None,
+                                    customized_BV=None, customized_num_warps=None):
+    """moda_v16.py:498-633.  ``customized_BT`` is the chunk size in query rows (default 64)."""
+    assert g_cumsum is None, "g_cumsum is not supported in this version"
+    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    assert q.shape[2] == k.shape[2], "Implicit head-dimension GQA is not allowed."
+    cb = _chunk_tokens(moda_group_num, customized_BT)
+    return _raw_fwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, scale, moda_group_num, cb)
+
+
+def parallel_moda_chunk_visible_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None,
+                                    cached_k=None, cached_v=None, moda_group_num=1, customized_BT=None,
+                                    customized_BS=None, customized_BK=None, customized_BV=None,
+                                    customized_num_warps=None):
+    """moda_v16.py:2099-2343."""
+    assert g_cumsum is None, "g_cumsum is not supported in this version"
+    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    cb = _chunk_tokens(moda_group_num, customized_BT)
+    dq, dk, dv, dkd, dvd = _raw_bwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, o, lse, do, scale,
+                                    moda_group_num, cb)
+    return dq, dk, dv, None, dkd, dvd
+
+
+class ParallelMixtureOfDepthAttentionChunkVisibleFunction(torch.autograd.Function):
+    """moda_v16.py:3456-3493 (9 inputs)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, q, k, v, g, scale, cu_seqlens, cached_k=None, cached_v=None, moda_group_num=1,
+                customized_BT=None):
+        o, lse = _autograd_forward(ctx, parallel_moda_chunk_visible_fwd, q, k, v, g, scale, cu_seqlens, cached_k,
+                                   cached_v, moda_group_num, customized_BT=customized_BT)
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, do, dlse_unused):
+        dq, dk, dv, dkd, dvd = _autograd_backward(ctx, parallel_moda_chunk_visible_bwd, do)
+        return dq, dk, dv, None, None, None, dkd, dvd, None, None
+
+
+def parallel_moda_chunk_visible(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_seqlens=None,
+                                moda_group_num=1, head_first=False, need_lse=False, return_depth_grads=True,
+                                warn_shape=True, customized_BT=None, customized_BS=None, customized_BT_backward=None,
+                                customized_BS_backward=None):
+    """Chunk-visible MoDA; signature of moda_v16.py:3614-3632.  A query of base
+    token ``t`` additionally sees the depth slots of tokens
+    ``floor(t/Cb)*Cb .. t`` with ``Cb = customized_BT // moda_group_num``
+    (``customized_BT`` defaults to 64 query rows)."""
+    q, k, v, g, cached_k, cached_v, scale = _prepare_inputs(
+        "parallel_moda_chunk_visible", q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first,
+        return_depth_grads, warn_shape)
+    o, lse = ParallelMixtureOfDepthAttentionChunkVisibleFunction.apply(
+        q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, customized_BT)
+    return (o, lse) if need_lse else o
+
+
+# ---------------------------------------------------------------------------
+# FDA (depth-only) -- fda_v12.py
+# ---------------------------------------------------------------------------
+def parallel_fda_fwd(q, g_cumsum, scale, cu_seqlens=None, cached_k=None, cached_v=None, moda_group_num=1,
+                     customized_BT=None, customized_BS=None, customized_BK=None, customized_BV=None,
+                     customized_num_warps=None):
+    """fda_v12.py:261-400.  Returns ``(o, lse)``."""
+    assert g_cumsum is None, "g_cumsum is not supported in this version"
+    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    assert cached_k is not None and cached_v is not None, "Flash Depth Attention requires cached_k/cached_v"
+    _assert_group_tile(moda_group_num)
+    return _raw_fwd(_lib.DEPTH_ONLY, q, None, None, cached_k, cached_v, scale, moda_group_num)
+
+
+def parallel_fda_bwd(q, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None, cached_k=None,
+                     cached_v=None, moda_group_num=1, customized_BT=None, customized_BS=None, customized_BK=None,
+                     customized_BV=None, customized_num_warps=None, group_bs=None, group_warps=None, depth_bs=None,
+                     depth_warps=None):
+    """fda_v12.py:881-1135.  Returns ``(dq, dg_cumsum=None, d_cached_k, d_cached_v)``."""
+    assert g_cumsum is None, "g_cumsum is not supported in this version"
+    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    dq, _, _, dkd, dvd = _raw_bwd(_lib.DEPTH_ONLY, q, None, None, cached_k, cached_v, o, lse, do, scale,
+                                  moda_group_num)
+    return dq, None, dkd, dvd
+
+
+class ParallelFlashDepthAttentionFunction(torch.autograd.Function):
+    """fda_v12.py:1207-1338 (13 inputs; the k, v slots must be None)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, q, k, v, g, scale, cu_seqlens, cached_k=None, cached_v=None, moda_group_num=1, group_bs=None,
+                group_warps=None, depth_bs=None, depth_warps=None):
+        assert g is None, "g is not supported in this version"
+        assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+        assert k is None and v is None, "Flash Depth Attention does not accept legacy k/v; pass None"
+        o, lse = parallel_fda_fwd(q, None, scale, None, cached_k, cached_v, moda_group_num)
+        ctx.save_for_backward(q, o, lse, cached_k, cached_v)
+        ctx.scale = scale
+        ctx.moda_group_num = moda_group_num
+        ctx.mark_non_differentiable(lse)
+        return o.to(q.dtype), lse
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, do, dlse_unused):
+        q, o, lse, cached_k, cached_v = ctx.saved_tensors
+        dq, _, dkd, dvd = parallel_fda_bwd(q, o, None, lse, do.to(o.dtype), ctx.scale, cached_k=cached_k,
+                                           cached_v=cached_v, moda_group_num=ctx.moda_group_num)
+        return dq.to(q), None, None, None, None, None, dkd, dvd, None, None, None, None, None
+
+
+def parallel_fda(q, k=None, v=None, g=None, cached_k=None, cached_v=None, scale=None, cu_seqlens=None,
+                 moda_group_num=1, head_first=False, need_lse=False, return_depth_grads=True, warn_shape=True,
+                 customized_BT=None, customized_BS=None, customized_BT_backward=None, customized_BS_backward=None,
+                 group_bs=None, group_warps=None, depth_bs=None, depth_warps=None):
+    """Depth-only attention; signature of fda_v12.py:1346-1368."""
+    assert k is None and v is None, "Flash Depth Attention does not accept legacy k/v; pass None"
+    if head_first:
+        q = q.transpose(1, 2)
+        if g is not None:
+            g = g.transpose(1, 2)
+        if cached_k is not None and cached_v is not None:
+            cached_k = cached_k.transpose(1, 2)
+            cached_v = cached_v.transpose(1, 2)
+    elif warn_shape and q.shape[1] < q.shape[2]:
+        warnings.warn(
+            f"[parallel_fda] detected seq_len({q.shape[1]}) < num_heads({q.shape[2]}). "
+            "input may be in head_first format while head_first=True is not set."
+        )
+    B, T_q, HQ, Kdim = q.shape
+    assert cached_k is not None and cached_v is not None, "Flash Depth Attention requires cached_k/cached_v"
+    assert moda_group_num > 0
+    assert T_q % moda_group_num == 0, "T_q must be divisible by moda_group_num"
+    T_kv = T_q // moda_group_num
+    H = cached_k.shape[2]
+    assert HQ == H, (
+        "Implicit head-dimension GQA is not allowed. "
+        "Please fold grouping only into `moda_group_num`: "
+        "use q.shape[2] == cached_k.shape[2] and set T_q = T_kv * moda_group_num."
+    )
+    if scale is None:
+        scale = Kdim ** -0.5
+    assert cached_k.shape[0] == B and cached_v.shape[0] == B
+    assert cached_k.shape[2] == H and cached_v.shape[2] == H, "cached_k/v head count mismatch"
+    assert cached_k.shape[1] % T_kv == 0, "cached_k time dimension must be T_kv * L"
+    L = cached_k.shape[1] // T_kv
+    assert L > 0
+    assert cached_v.shape[1] == T_kv * L, "cached_v shape mismatch"
+    if (cached_k.requires_grad or cached_v.requires_grad) and not return_depth_grads:
+        warnings.warn(
+            "cached_k/v requires gradients, but return_depth_grads=False. "
+            "Gradients are still computed and returned."
+        )
+    if g is not None:
+        assert g.shape[:3] == (B, T_q, HQ), "g must be [B,T_q,HQ]"
+    o, lse = ParallelFlashDepthAttentionFunction.apply(q, k, v, g, scale, cu_seqlens, cached_k, cached_v,
+                                                       moda_group_num, group_bs, group_warps, depth_bs, depth_warps)
+    return (o, lse) if need_lse else o
+
+
+# ---------------------------------------------------------------------------
+# plain causal attention with head-dim GQA -- fla/ops/attn/parallel.py
+# ---------------------------------------------------------------------------
+def parallel_attn_fwd(q, k, v, g_cumsum=None, scale=None, cu_seqlens=None):
+    """fla/ops/attn/parallel.py:443-503.  q ``[B,T,HQ,D]``, k/v ``[B,T,H,D]``; returns ``(o, lse)``."""
+    assert g_cumsum is None and cu_seqlens is None
+    assert q.shape[2] % k.shape[2] == 0, "HQ must be a multiple of H"
+    assert q.shape[1] == k.shape[1]
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    return _raw_fwd(_lib.PLAIN_GQA, q, k, v, None, None, scale, q.shape[2] // k.shape[2])
+
+
+def parallel_attn_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None):
+    """fla/ops/attn/parallel.py:522-629.  Returns ``(dq, dk, dv, dg=None)``."""
+    assert g_cumsum is None and cu_seqlens is None
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    dq, dk, dv, _, _ = _raw_bwd(_lib.PLAIN_GQA, q, k, v, None, None, o, lse, do, scale, q.shape[2] // k.shape[2])
+    return dq, dk, dv, None
+
+
+class ParallelAttentionFunction(torch.autograd.Function):
+    """fla/ops/attn/parallel.py:632-675."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, q, k, v, g, scale, cu_seqlens):
+        assert g is None, "g is not supported"
+        assert cu_seqlens is None, "cu_seqlens is not supported"
+        o, lse = parallel_attn_fwd(q, k, v, None, scale, None)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.scale = scale
+        return o.to(q.dtype)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, do):
+        q, k, v, o, lse = ctx.saved_tensors
+        dq, dk, dv, _ = parallel_attn_bwd(q, k, v, o, None, lse, do.to(o.dtype), ctx.scale)
+        return dq.to(q), dk.to(k), dv.to(v), None, None, None
+
+
+def parallel_attn(q, k, v, g=None, scale=None, cu_seqlens=None, head_first=False):
+    """Plain causal attention with head-dim GQA; signature of fla/ops/attn/parallel.py:678-686."""
+    if head_first:
+        raise DeprecationWarning(
+            "head_first is deprecated and will be removed in a future version. "
+            "Please use head_first=False for now instead."
+        )
+    if q.shape[1] < q.shape[2]:
+        warnings.warn(
+            f"Input tensor shape suggests potential format mismatch: seq_len ({q.shape[1]}) < num_heads ({q.shape[2]}). "
+        )
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    return ParallelAttentionFunction.apply(q, k, v, g, scale, cu_seqlens)
