@@ -109,6 +109,25 @@ int moda_hip_bwd(const moda_hip_desc* desc, const void* q, const void* k, const 
                  void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * moda_hip_bwd restricted to the stages named in `stages` (an OR of the values
+ * below); the stages of one backward must run in the order DELTA, DQ, DKV on
+ * one stream (DQ and DKV read the workspace DELTA writes).  Lets a caller skip
+ * dK/dV when only dQ is needed, or time the stages separately.  The reference
+ * launches the same three steps one after another (moda_v14.py:1609, 1658,
+ * 1698-1801).
+ */
+enum moda_hip_bwd_stage {
+  MODA_HIP_STAGE_DELTA = 1, /* delta = rowsum(o * do)                 */
+  MODA_HIP_STAGE_DQ = 2,    /* dq                                     */
+  MODA_HIP_STAGE_DKV = 4,   /* dk, dv and, with a depth stream, dkd, dvd */
+  MODA_HIP_STAGE_ALL = 7
+};
+int moda_hip_bwd_stages(const moda_hip_desc* desc, const void* q, const void* k, const void* v,
+                        const void* kd, const void* vd, const void* o, const float* lse, const void* d_o,
+                        void* dq, void* dk, void* dv, void* dkd, void* dvd,
+                        void* workspace, size_t workspace_bytes, int stages, void* stream);
+
+/*
  * Depth-KV reorganisation.  Replaces the caller-side
  * torch.stack(dim=2).reshape(B, T*L, H, D).contiguous() of
  * vision_tasks/deit/models.py:361-375 (one call per tensor, K or V).

@@ -15,11 +15,13 @@ LIB_PATH = os.path.join(_HERE, "libmoda_hip.so")
 
 BF16, FP16, FP32 = 0, 1, 2
 CAUSAL, NONCAUSAL, CHUNK_VISIBLE, DEPTH_ONLY, PLAIN_GQA = 0, 1, 2, 3, 4
+STAGE_DELTA, STAGE_DQ, STAGE_DKV, STAGE_ALL = 1, 2, 4, 7
 
 EXPORTS = (
     "moda_hip_fwd",
     "moda_hip_bwd_workspace_bytes",
     "moda_hip_bwd",
+    "moda_hip_bwd_stages",
     "moda_hip_depth_reorg_fwd",
     "moda_hip_depth_reorg_bwd",
     "moda_hip_strerror",
@@ -86,6 +88,8 @@ def load():
     lib.moda_hip_bwd_workspace_bytes.argtypes = [POINTER(Desc)]
     lib.moda_hip_bwd.restype = c_int
     lib.moda_hip_bwd.argtypes = [POINTER(Desc)] + [vp] * 14 + [c_size_t, vp]
+    lib.moda_hip_bwd_stages.restype = c_int
+    lib.moda_hip_bwd_stages.argtypes = [POINTER(Desc)] + [vp] * 14 + [c_size_t, c_int, vp]
     lib.moda_hip_depth_reorg_fwd.restype = c_int
     lib.moda_hip_depth_reorg_fwd.argtypes = [POINTER(vp), c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                              c_int64, c_int32, vp, vp]

@@ -192,6 +192,14 @@ __global__ __launch_bounds__(256) void dq_kernel(const KArgs a) {
 }
 
 template <typename T, int HD>
+hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
+  if (a.Tq == 0 || a.B * a.Hq == 0) return hipSuccess;
+  constexpr int RPB = 256 / (HD / 8);
+  hipLaunchKernelGGL((delta_kernel<T, HD>), dim3((a.Tq + RPB - 1) / RPB, a.B * a.Hq), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+template <typename T, int HD>
 hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = 4 * 64 * HD * sizeof(uint16_t);
   static bool attr_done = false;
@@ -201,14 +209,18 @@ hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  if (a.Tq == 0 || a.B * a.Hq == 0) return hipSuccess;
-  constexpr int RPB = 256 / (HD / 8);
-  hipLaunchKernelGGL((delta_kernel<T, HD>), dim3((a.Tq + RPB - 1) / RPB, a.B * a.Hq), dim3(256), 0, stream, a);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
   const int64_t nblk = (int64_t)a.nqt * a.B * a.Hq;
+  if (nblk == 0) return hipSuccess;
   hipLaunchKernelGGL((dq_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), smem, stream, a);
   return hipGetLastError();
+}
+
+hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream) {
+  if (dtype == 0 && hd == 128) return launch_delta_t<BF16, 128>(a, stream);
+  if (dtype == 0 && hd == 64) return launch_delta_t<BF16, 64>(a, stream);
+  if (dtype == 1 && hd == 128) return launch_delta_t<FP16, 128>(a, stream);
+  if (dtype == 1 && hd == 64) return launch_delta_t<FP16, 64>(a, stream);
+  return hipErrorInvalidValue;
 }
 
 hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream) {

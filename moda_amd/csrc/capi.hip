@@ -8,6 +8,7 @@
 
 namespace moda {
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream);
+hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_generic(const KArgs& a, int dtype, int D, int which, hipStream_t stream);
@@ -141,9 +142,18 @@ size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* d) {
 int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
                  const void* vd, const void* o, const float* lse, const void* d_o, void* dq, void* dk, void* dv,
                  void* dkd, void* dvd, void* workspace, size_t workspace_bytes, void* stream) {
+  return moda_hip_bwd_stages(d, q, k, v, kd, vd, o, lse, d_o, dq, dk, dv, dkd, dvd, workspace, workspace_bytes,
+                             MODA_HIP_STAGE_ALL, stream);
+}
+
+int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
+                        const void* vd, const void* o, const float* lse, const void* d_o, void* dq, void* dk,
+                        void* dv, void* dkd, void* dvd, void* workspace, size_t workspace_bytes, int stages,
+                        void* stream) {
   KArgs a;
   int rc = fill_geometry(d, a);
   if (rc) return rc;
+  if (stages < 0 || stages > MODA_HIP_STAGE_ALL) return MODA_HIP_EINVAL;
   const int es = elem_size(d->dtype);
   const bool have_rows = (int64_t)a.B * a.Tq * a.Hq > 0;
   if (have_rows) {
@@ -208,13 +218,15 @@ int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const voi
   a.sdkd = cvt(d->dkd);
   a.sdvd = cvt(d->dvd);
   hipStream_t s = (hipStream_t)stream;
-  hipError_t e;
+  hipError_t e = hipSuccess;
   if (use_mfma(d)) {
-    e = moda::launch_dq(a, d->dtype, (int)d->D, s);
-    if (e == hipSuccess) e = moda::launch_dkv(a, d->dtype, (int)d->D, s);
+    if (stages & MODA_HIP_STAGE_DELTA) e = moda::launch_delta(a, d->dtype, (int)d->D, s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ)) e = moda::launch_dq(a, d->dtype, (int)d->D, s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_dkv(a, d->dtype, (int)d->D, s);
   } else {
-    e = moda::launch_generic(a, d->dtype, (int)d->D, 1, s);
-    if (e == hipSuccess) e = moda::launch_generic(a, d->dtype, (int)d->D, 2, s);
+    // the generic kernels recompute delta inline; the DELTA stage is a no-op for them
+    if (stages & MODA_HIP_STAGE_DQ) e = moda::launch_generic(a, d->dtype, (int)d->D, 1, s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_generic(a, d->dtype, (int)d->D, 2, s);
   }
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }

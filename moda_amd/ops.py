@@ -132,29 +132,37 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0):
     return o, lse
 
 
-def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0):
-    """Launch the backward kernels. Returns (dq, dk, dv, dkd, dvd)."""
+def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages=_lib.STAGE_ALL, out=None, ws=None):
+    """Launch the backward kernels. Returns (dq, dk, dv, dkd, dvd).
+
+    ``stages`` selects a subset of {delta, dq, dk/dv}; ``out`` (a previous return
+    value) and ``ws`` (a workspace tensor) let the caller reuse buffers across calls."""
     _check_device(q)
     _same_dtype(q, k, v, kd, vd, o, do)
     q, k, v, kd, vd, o, do = map(_usable, (q, k, v, kd, vd, o, do))
     lse = lse.contiguous()
     T = q.shape[1] // G if mode == _lib.DEPTH_ONLY else k.shape[1]
     L = (kd.shape[1] // T) if (kd is not None and T > 0) else 0
-    dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    dk = torch.empty(k.shape, dtype=k.dtype, device=q.device) if k is not None else None
-    dv = torch.empty(v.shape, dtype=v.dtype, device=q.device) if v is not None else None
-    dkd = torch.empty(kd.shape, dtype=kd.dtype, device=q.device) if kd is not None else None
-    dvd = torch.empty(vd.shape, dtype=vd.dtype, device=q.device) if vd is not None else None
+    if out is not None:
+        dq, dk, dv, dkd, dvd = out
+    else:
+        dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        dk = torch.empty(k.shape, dtype=k.dtype, device=q.device) if k is not None else None
+        dv = torch.empty(v.shape, dtype=v.dtype, device=q.device) if v is not None else None
+        dkd = torch.empty(kd.shape, dtype=kd.dtype, device=q.device) if kd is not None else None
+        dvd = torch.empty(vd.shape, dtype=vd.dtype, device=q.device) if vd is not None else None
     kd_a, vd_a, dkd_a, dvd_a = (kd, vd, dkd, dvd) if L > 0 else (None, None, None, None)
     d = _desc(mode, q, k, v, kd_a, vd_a, G, L, chunk_tokens, scale, o=o, do=do, dq=dq, dk=dk, dv=dv, dkd=dkd_a,
               dvd=dvd_a)
     lib = _lib.load()
     nbytes = lib.moda_hip_bwd_workspace_bytes(ctypes.byref(d))
-    ws = torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=q.device)
+    if ws is None:
+        ws = torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
-        rc = lib.moda_hip_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kd_a), _ptr(vd_a), _ptr(o), _ptr(lse),
-                              _ptr(do), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dkd_a), _ptr(dvd_a), _ptr(ws),
-                              ctypes.c_size_t(ws.numel()), _stream(q))
+        rc = lib.moda_hip_bwd_stages(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kd_a), _ptr(vd_a), _ptr(o),
+                                     _ptr(lse), _ptr(do), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dkd_a), _ptr(dvd_a),
+                                     _ptr(ws), ctypes.c_size_t(ws.numel() * ws.element_size()), int(stages),
+                                     _stream(q))
     _lib.check(rc, "moda_hip_bwd")
     return dq, dk, dv, dkd, dvd
 

@@ -176,12 +176,11 @@ def moda_dense(
     use_depth = kd is not None and vd is not None
     if mode == "depth_only":
         assert use_depth
-        T = (Tq_in // G) if rows is None else None
-        L = None
-    if mode != "depth_only":
+        if rows is not None:
+            raise ValueError("rows= is not supported for depth_only (T is inferred from the full q)")
+        T = Tq_in // G
+    else:
         T = k.shape[1]
-    elif rows is not None:
-        raise ValueError("rows= needs T; pass k=None only with full q")
     L = kd.shape[1] // T if use_depth else 0
     if scale is None:
         scale = 1.0 / math.sqrt(D)
@@ -240,14 +239,16 @@ def moda_rows_subset(inp, rows: torch.Tensor, scale, G, mode, chunk_tokens=0, dt
 # --------------------------------------------------------------------------
 @torch.no_grad()
 def moda_blockwise_fwd_bwd(inp, scale, G, mode, chunk_tokens=0, block_rows=4096, dtype=torch.float32,
-                           o_round_dtype=None):
+                           o_round_dtype=None, token_range=None):
     """Tiled evaluation for long sequences; runs on whatever device ``inp`` is on.
 
     Uses the closed-form gradients of softmax attention
     (``ds = p * (dp - delta)``, ``delta = sum(o * do)``) instead of autograd so
     that only ``block_rows x keys`` scores are alive at a time.  ``o_round_dtype``
     optionally rounds ``o`` before ``delta`` as the kernels do (moda_v14.py:525-539
-    reads the stored, rounded ``o``).
+    reads the stored, rounded ``o``).  ``token_range=(a, b)`` evaluates only the query rows of tokens
+    ``a <= t < b`` (outputs of other rows are left unset, key gradients hold only those rows'
+    contributions); used to time a bounded sample of a large workload.
     """
     q, k, v, kd, vd, do = (inp.get(n) for n in ("q", "k", "v", "kd", "vd", "do"))
     B, Tq, H, D = q.shape
@@ -273,8 +274,11 @@ def moda_blockwise_fwd_bwd(inp, scale, G, mode, chunk_tokens=0, block_rows=4096,
     step_tok = max(1, block_rows // G)
     if mode == "chunk_visible":
         step_tok = max(chunk_tokens, (step_tok // chunk_tokens) * chunk_tokens)
-    for t0 in range(0, T, step_tok):
-        t1 = min(T, t0 + step_tok)
+    tok_a, tok_b = (0, T) if token_range is None else token_range
+    if mode == "chunk_visible":
+        assert tok_a % chunk_tokens == 0
+    for t0 in range(tok_a, tok_b, step_tok):
+        t1 = min(tok_b, t0 + step_tok)
         r0, r1 = t0 * G, t1 * G
         rows = torch.arange(r0, r1, device=dev)
         tok = rows // G

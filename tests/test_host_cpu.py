@@ -1,0 +1,153 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads and exports
+every symbol the header declares, the ctypes mirror of the descriptor matches,
+and the host functions keep the reference's argument contract
+(moda_v14.py:2834-2871, fda_v12.py:1370-1437).  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_functions():
+    text = open(os.path.join(ROOT, "include", "moda_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(moda_hip_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from moda_amd import _lib
+
+    lib = _lib.load()
+    names = _header_functions()
+    assert set(names) == set(_lib.EXPORTS)
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_descriptor_layout_and_version():
+    from moda_amd import _lib
+
+    lib = _lib.load()
+    assert lib.moda_hip_version() == 100
+    assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24
+    assert _lib.Desc.q.offset == 80
+    # a descriptor with the wrong struct_size is rejected without touching any device
+    d = _lib.Desc()
+    d.struct_size = 12
+    assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(d)) == 0
+    assert lib.moda_hip_fwd(ctypes.byref(d), None, None, None, None, None, None, None, None) == -1
+    assert b"invalid" in lib.moda_hip_strerror(-1)
+
+
+def test_descriptor_validation_codes():
+    from moda_amd import _lib
+
+    lib = _lib.load()
+
+    def desc(**kw):
+        d = _lib.Desc()
+        d.struct_size = ctypes.sizeof(_lib.Desc)
+        d.dtype, d.mode = _lib.BF16, _lib.CAUSAL
+        d.B, d.T, d.H, d.G, d.D, d.L = 1, 8, 1, 1, 64, 0
+        d.scale = 1.0
+        for k, v in kw.items():
+            setattr(d, k, v)
+        return d
+
+    assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc())) == 8 * 4
+    assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc(G=4, H=2, B=3))) == 3 * 2 * 32 * 4
+    assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc(mode=_lib.PLAIN_GQA, G=4, H=2))) == 8 * 8 * 4
+    null = None
+    # missing q pointer
+    assert lib.moda_hip_fwd(ctypes.byref(desc()), null, null, null, null, null, null, null, null) == -1
+    # unsupported head dim
+    assert lib.moda_hip_fwd(ctypes.byref(desc(D=512)), null, null, null, null, null, null, null, null) == -2
+    # depth-only without depth slots, plain GQA with depth slots, chunk-visible without chunk size
+    assert lib.moda_hip_fwd(ctypes.byref(desc(mode=_lib.DEPTH_ONLY)), null, null, null, null, null, null, null, null) == -1
+    assert lib.moda_hip_fwd(ctypes.byref(desc(mode=_lib.PLAIN_GQA, L=2)), null, null, null, null, null, null, null, null) == -1
+    assert lib.moda_hip_fwd(ctypes.byref(desc(mode=_lib.CHUNK_VISIBLE, L=2)), null, null, null, null, null, null, null, null) == -1
+    # empty problem is a successful no-op
+    assert lib.moda_hip_fwd(ctypes.byref(desc(T=0)), null, null, null, null, null, null, null, null) == 0
+    # misaligned pointer (never dereferenced: alignment is checked first)
+    bogus = ctypes.c_void_p(0x1008)
+    ok = ctypes.c_void_p(0x1000)
+    assert lib.moda_hip_fwd(ctypes.byref(desc()), bogus, ok, ok, null, null, ok, ok, null) == -3
+    # reorg argument checks
+    arr = (ctypes.c_void_p * 1)(0x1000)
+    assert lib.moda_hip_depth_reorg_fwd(arr, 1, 3, 3, 1, 4, 1, 64, _lib.BF16, ok, null) == -1  # slot out of range
+    assert lib.moda_hip_depth_reorg_fwd(arr, 0, 0, 3, 1, 4, 1, 64, _lib.BF16, ok, null) == 0   # nothing to do
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from moda_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmoda_hip.so")
+    with pytest.raises(_lib.MissingLibraryError):
+        _lib.load()
+
+
+def test_cpu_tensors_are_rejected():
+    import moda_amd
+
+    q = torch.zeros(1, 8, 1, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        moda_amd.parallel_moda(q, q, q)
+
+
+def test_argument_contract_matches_reference():
+    import moda_amd
+
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16)
+    # implicit head-dim GQA is refused (moda_v14.py:2839-2843)
+    with pytest.raises(AssertionError, match="Implicit head-dimension GQA"):
+        moda_amd.parallel_moda(z(1, 8, 4, 64), z(1, 8, 2, 64), z(1, 8, 2, 64))
+    # T_q must be T_kv * G (moda_v14.py:2847-2852)
+    with pytest.raises(AssertionError, match="T_q must equal T_kv"):
+        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), moda_group_num=2)
+    with pytest.raises(AssertionError, match="moda_group_num=1"):
+        moda_amd.parallel_moda(z(1, 16, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64))
+    # depth cache shape checks (moda_v14.py:2856-2862)
+    with pytest.raises(AssertionError, match="T_kv \\* L"):
+        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), cached_k=z(1, 12, 2, 64),
+                               cached_v=z(1, 12, 2, 64))
+    with pytest.raises(AssertionError, match="head count"):
+        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), cached_k=z(1, 16, 1, 64),
+                               cached_v=z(1, 16, 1, 64))
+    # g / cu_seqlens are unsupported (moda_v14.py:2672-2673)
+    with pytest.raises(AssertionError, match="g is not supported"):
+        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), g=torch.zeros(1, 8, 2))
+    with pytest.raises(AssertionError, match="cu_seqlens is not supported"):
+        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), cu_seqlens=torch.tensor([0, 8]))
+    # group size must divide the query tile (moda_v14.py:476-478)
+    with pytest.raises(AssertionError, match="BT % moda_group_num"):
+        moda_amd.parallel_moda(z(1, 24, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), moda_group_num=3)
+    # FDA (fda_v12.py:1370-1372, 1391-1393)
+    with pytest.raises(AssertionError, match="does not accept legacy k/v"):
+        moda_amd.parallel_fda(z(1, 8, 2, 64), k=z(1, 8, 2, 64), v=z(1, 8, 2, 64), cached_k=z(1, 16, 2, 64),
+                              cached_v=z(1, 16, 2, 64))
+    with pytest.raises(AssertionError, match="requires cached_k/cached_v"):
+        moda_amd.parallel_fda(z(1, 8, 2, 64))
+    # seq_len < num_heads warning (moda_v14.py:2828-2832)
+    with pytest.warns(UserWarning, match="head_first"):
+        with pytest.raises(RuntimeError):
+            moda_amd.parallel_moda(z(1, 2, 4, 64), z(1, 2, 4, 64), z(1, 2, 4, 64))
+
+
+def test_compat_package_reexports():
+    import sys
+
+    sys.path.insert(0, os.path.join(ROOT, "moda_amd", "compat"))
+    try:
+        from fla.ops.moda import parallel_moda, parallel_moda_chunk_visible  # noqa: F401
+        import moda_amd
+
+        assert parallel_moda is moda_amd.parallel_moda
+    finally:
+        sys.path.pop(0)
+        for m in [m for m in sys.modules if m == "fla" or m.startswith("fla.")]:
+            del sys.modules[m]
