@@ -19,10 +19,10 @@ template <typename T, int HD>
 __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
   constexpr int BN = 128, BM = 64, KK = HD / 16, DB = HD / 32;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  uint16_t* smem = reinterpret_cast<uint16_t*>(smem_raw);
-  uint16_t* Qs[2] = {smem, smem + BM * HD};
-  uint16_t* dOs[2] = {smem + 2 * BM * HD, smem + 3 * BM * HD};
-  float* stat = reinterpret_cast<float*>(smem + 4 * BM * HD);  // [2][2][BM]: lse, delta per stage
+  lds_ptr smem = (lds_ptr)smem_raw;
+  lds_ptr Qs[2] = {smem, smem + BM * HD};
+  lds_ptr dOs[2] = {smem + 2 * BM * HD, smem + 3 * BM * HD};
+  MODA_LDS float* stat = (MODA_LDS float*)(smem + 4 * BM * HD);  // [2][2][BM]: lse, delta per stage
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
   const int BHk = a.B * a.Hkv;
@@ -68,6 +68,8 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
   const int niter = nqt * a.hdiv;
 
   TileLoader<HD, BM, 256> ldq, ldo;
+  ldq.init(tid);
+  ldo.init(tid);
   float st_reg = 0.f;
   auto issue = [&](int it) {
     const int gh = it / nqt;
@@ -84,8 +86,8 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
     }
   };
   auto commit = [&](int stage) {
-    ldq.store(Qs[stage], tid);
-    ldo.store(dOs[stage], tid);
+    ldq.store(Qs[stage]);
+    ldo.store(dOs[stage]);
     if (tid < 2 * BM) stat[stage * 2 * BM + tid] = st_reg;
   };
 
@@ -113,8 +115,8 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
     if (__any(touches)) {
       const bool full = (qlo <= q0) && (qhi >= q0 + BM);
       const bool need_mask = !__all(full);
-      const float* lse_s = stat + cur * 2 * BM;
-      const float* del_s = lse_s + BM;
+      MODA_LDS const float* lse_s = stat + cur * 2 * BM;
+      MODA_LDS const float* del_s = lse_s + BM;
       f32x16 s[2], dp[2];
 #pragma unroll
       for (int bb = 0; bb < 2; bb++) {
@@ -134,8 +136,8 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
 #pragma unroll
         for (int i4 = 0; i4 < 4; i4++) {
           const int row0 = 32 * bb + 8 * i4 + 4 * g;
-          const f32x4 lv = *reinterpret_cast<const f32x4*>(lse_s + row0);
-          const f32x4 dl = *reinterpret_cast<const f32x4*>(del_s + row0);
+          const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
+          const f32x4 dl = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + row0);
 #pragma unroll
           for (int j = 0; j < 4; j++) {
             const int i = 4 * i4 + j;

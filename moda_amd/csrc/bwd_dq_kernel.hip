@@ -36,12 +36,12 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a) {
 }
 
 template <typename T, int HD>
-__global__ __launch_bounds__(256) void dq_kernel(const KArgs a) {
+__global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
   constexpr int BM = 128, BN = 64, KK = HD / 16, DB = HD / 32;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  uint16_t* smem = reinterpret_cast<uint16_t*>(smem_raw);
-  uint16_t* Ks[2] = {smem, smem + BN * HD};
-  uint16_t* Vs[2] = {smem + 2 * BN * HD, smem + 3 * BN * HD};
+  lds_ptr smem = (lds_ptr)smem_raw;
+  lds_ptr Ks[2] = {smem, smem + BN * HD};
+  lds_ptr Vs[2] = {smem + 2 * BN * HD, smem + 3 * BN * HD};
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
   const int BH = a.B * a.Hq;
@@ -98,6 +98,8 @@ __global__ __launch_bounds__(256) void dq_kernel(const KArgs a) {
   const int TL = a.T * a.L;
 
   TileLoader<HD, BN, 256> ldk, ldv;
+  ldk.init(tid);
+  ldv.init(tid);
   auto issue = [&](int it) {
     if (it < n_seq) {
       ldk.load(kb, a.sk.t, it * BN, a.T, tid);
@@ -118,8 +120,8 @@ __global__ __launch_bounds__(256) void dq_kernel(const KArgs a) {
 
   if (ntiles > 0) {
     issue(0);
-    ldk.store(Ks[0], tid);
-    ldv.store(Vs[0], tid);
+    ldk.store(Ks[0]);
+    ldv.store(Vs[0]);
   }
   __syncthreads();
 
@@ -171,8 +173,8 @@ __global__ __launch_bounds__(256) void dq_kernel(const KArgs a) {
     }
 
     if (it + 1 < ntiles) {
-      ldk.store(Ks[cur ^ 1], tid);
-      ldv.store(Vs[cur ^ 1], tid);
+      ldk.store(Ks[cur ^ 1]);
+      ldv.store(Vs[cur ^ 1]);
     }
     __syncthreads();
   }

@@ -15,12 +15,12 @@
 namespace moda {
 
 template <typename T, int HD>
-__global__ __launch_bounds__(256) void fwd_kernel(const KArgs a) {
+__global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
   constexpr int BM = 128, BN = 64, KK = HD / 16, DB = HD / 32;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  uint16_t* smem = reinterpret_cast<uint16_t*>(smem_raw);
-  uint16_t* Ks[2] = {smem, smem + BN * HD};
-  uint16_t* Vs[2] = {smem + 2 * BN * HD, smem + 3 * BN * HD};
+  lds_ptr smem = (lds_ptr)smem_raw;
+  lds_ptr Ks[2] = {smem, smem + BN * HD};
+  lds_ptr Vs[2] = {smem + 2 * BN * HD, smem + 3 * BN * HD};
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
   const int BH = a.B * a.Hq;
@@ -72,6 +72,8 @@ __global__ __launch_bounds__(256) void fwd_kernel(const KArgs a) {
   const int TL = a.T * a.L;
 
   TileLoader<HD, BN, 256> ldk, ldv;
+  ldk.init(tid);
+  ldv.init(tid);
   auto issue = [&](int it) {
     if (it < n_seq) {
       ldk.load(kb, a.sk.t, it * BN, a.T, tid);
@@ -93,8 +95,8 @@ __global__ __launch_bounds__(256) void fwd_kernel(const KArgs a) {
 
   if (ntiles > 0) {
     issue(0);
-    ldk.store(Ks[0], tid);
-    ldv.store(Vs[0], tid);
+    ldk.store(Ks[0]);
+    ldv.store(Vs[0]);
   }
   __syncthreads();
 
@@ -119,6 +121,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const KArgs a) {
         for (int kk = 0; kk < KK; kk++)
           s[bb] = mfma32<T>(lds_row_operand<HD>(Ks[cur], 32 * bb, kk, lane), Qr[kk], s[bb]);
       }
+      // row maximum of the raw scores (scale > 0, so it commutes with the max)
       float mx = kNegInf;
       if (need_mask) {
 #pragma unroll
@@ -126,7 +129,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const KArgs a) {
 #pragma unroll
           for (int i = 0; i < 16; i++) {
             const int c = col0 + 32 * bb + acc_row(i, g);
-            const float x = (c >= lo && c < hi) ? s[bb][i] * sc : kNegInf;
+            const float x = (c >= lo && c < hi) ? s[bb][i] : kNegInf;
             s[bb][i] = x;
             mx = fmaxf(mx, x);
           }
@@ -134,32 +137,34 @@ __global__ __launch_bounds__(256) void fwd_kernel(const KArgs a) {
 #pragma unroll
         for (int bb = 0; bb < 2; bb++)
 #pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const float x = s[bb][i] * sc;
-            s[bb][i] = x;
-            mx = fmaxf(mx, x);
-          }
+          for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[bb][i]);
       }
-      mx = fmaxf(mx, xor32(mx));
-      const float m_new = fmaxf(m, mx);
-      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-      const float alpha = fast_exp2(m - m_safe);
+      mx = fmaxf(mx, xor32(mx)) * sc;
+      // The exponent reference m only moves when some row's maximum outgrows it by more than 2^8:
+      // p stays <= 256, exact in fp32 accumulation and harmless in the 16-bit P, and the
+      // rescale of O is skipped on almost every tile.
+      if (__any(mx > m + 8.f)) {
+        const float m_new = fmaxf(m, mx);
+        const float alpha = fast_exp2(m - ((m_new == kNegInf) ? 0.f : m_new));
+        l *= alpha;
+        m = m_new;
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) o[d][i] *= alpha;
+      }
+      const float neg_m = (m == kNegInf) ? 0.f : -m;
       float rs = 0.f;
 #pragma unroll
       for (int bb = 0; bb < 2; bb++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          const float p = fast_exp2(s[bb][i] - m_safe);
+          const float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m));
           s[bb][i] = p;
           rs += p;
         }
       rs += xor32(rs);
-      l = l * alpha + rs;
-      m = m_new;
-#pragma unroll
-      for (int d = 0; d < DB; d++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o[d][i] *= alpha;
+      l += rs;
       i32x4 P[4];
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
@@ -170,8 +175,8 @@ __global__ __launch_bounds__(256) void fwd_kernel(const KArgs a) {
     }
 
     if (it + 1 < ntiles) {
-      ldk.store(Ks[cur ^ 1], tid);
-      ldv.store(Vs[cur ^ 1], tid);
+      ldk.store(Ks[cur ^ 1]);
+      ldv.store(Vs[cur ^ 1]);
     }
     __syncthreads();
   }

@@ -31,6 +31,8 @@ struct FP16 {
 };
 
 #define MODA_LDS __attribute__((address_space(3)))
+typedef MODA_LDS uint16_t* lds_ptr;        // LDS tile pointer (32-bit, address space 3)
+typedef MODA_LDS const uint16_t* lds_cptr;
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegInf = -__builtin_huge_valf();
@@ -104,10 +106,10 @@ struct Tile {
 // Row operand: lane (n, g) gets elements [16*kk + 8g, +8) of row (row0 + n).
 // Serves as MFMA A (M = tile rows) or B (N = tile rows) with K = head dim.
 template <int HD>
-__device__ __forceinline__ i32x4 lds_row_operand(const uint16_t* tile, int row0, int kk, int lane) {
+__device__ __forceinline__ i32x4 lds_row_operand(lds_cptr tile, int row0, int kk, int lane) {
   const int n = lane & 31, g = lane >> 5;
-  const uint16_t* p = tile + Tile<HD>::off(row0 + n, 2 * kk + g);
-  return *reinterpret_cast<const i32x4*>(p);
+  lds_cptr p = tile + Tile<HD>::off(row0 + n, 2 * kk + g);
+  return *reinterpret_cast<MODA_LDS const i32x4*>(p);
 }
 
 // Transposed operand: lane (n, g) gets, for head-dim column d = 32*dblk + n,
@@ -118,13 +120,13 @@ __device__ __forceinline__ i32x4 lds_row_operand(const uint16_t* tile, int row0,
 // r supplies the address of 4 consecutive elements; result lane i receives
 // element (i & 3) of source lanes 4j + (i >> 2), j = 0..3.
 template <int HD>
-__device__ __forceinline__ i32x4 lds_tr_operand(const uint16_t* tile, int rb, int dblk, int lane) {
+__device__ __forceinline__ i32x4 lds_tr_operand(lds_cptr tile, int rb, int dblk, int lane) {
   const int g = lane >> 5;
   const int r16 = lane & 15;
   const int row = rb + 4 * g + (r16 >> 2);
   const int dcol = 32 * dblk + ((lane >> 4) & 1) * 16 + (r16 & 3) * 4;
-  const uint16_t* p0 = tile + Tile<HD>::off(row, dcol >> 3) + (dcol & 7);
-  const uint16_t* p1 = tile + Tile<HD>::off(row + 8, dcol >> 3) + (dcol & 7);
+  lds_cptr p0 = tile + Tile<HD>::off(row, dcol >> 3) + (dcol & 7);
+  lds_cptr p1 = tile + Tile<HD>::off(row + 8, dcol >> 3) + (dcol & 7);
   s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(p0));
   s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(p1));
   i32x2 l2 = __builtin_bit_cast(i32x2, lo);
@@ -137,35 +139,41 @@ __device__ __forceinline__ i32x4 lds_tr_operand(const uint16_t* tile, int rb, in
   return r;
 }
 
+// Raw buffer resource over `nbytes` bytes at `base` (wave-uniform): loads past the end return zero.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t nbytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)nbytes, 0x00020000);
+}
+
 // Cooperative global -> register -> LDS staging of a ROWS x HD tile by NT threads.
-// Rows outside [0, nrows) relative to `base` read as zero.
+// Global side: buffer loads with hardware range checking (rows past the end of
+// the source read as zero, no branches) and all per-pass address increments in
+// the scalar offset.  LDS side: swizzled 16-byte stores at a per-thread base
+// plus compile-time offsets.
 template <int HD, int ROWS, int NT>
 struct TileLoader {
-  static constexpr int CH = HD / 8;
-  static constexpr int N = (ROWS * CH) / NT;  // 16-byte chunks per thread
-  static_assert((ROWS * CH) % NT == 0, "tile must divide evenly");
+  static constexpr int CH = HD / 8;            // 16-byte chunks per row
+  static constexpr int RPP = NT / CH;          // rows covered per pass
+  static constexpr int N = ROWS / RPP;         // passes = 16-byte chunks per thread
+  static_assert(NT % CH == 0 && ROWS % RPP == 0 && RPP % 16 == 0, "tile must divide evenly");
   i32x4 r[N];
+  int lds_off;  // element offset of this thread's chunk in pass 0
 
-  // src points at row 0 of the (batch, head) slice; rows outside [0, row_end) are zero-filled
-  __device__ __forceinline__ void load(const uint16_t* src, int64_t row_stride, int64_t row0, int64_t row_end,
-                                       int tid) {
+  __device__ __forceinline__ void init(int tid) { lds_off = Tile<HD>::off(tid / CH, tid % CH); }
+
+  // src: row 0 of the (batch, head) slice; rows [row0, row0 + ROWS) are fetched, rows >= row_end read as zero.
+  __device__ __forceinline__ void load(const uint16_t* src, int64_t row_stride, int row0, int row_end, int tid) {
+    const int rows_left = row_end - row0;
+    const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
+    const uint32_t nbytes = rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(src + (int64_t)row0 * row_stride, nbytes);
+    const int voff = (tid / CH) * (int)stride_bytes + (tid % CH) * 16;
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-      const int id = tid + i * NT;
-      const int row = id / CH, ch = id % CH;
-      const int64_t gr = row0 + row;
-      i32x4 v = {0, 0, 0, 0};
-      if (gr >= 0 && gr < row_end) v = *reinterpret_cast<const i32x4*>(src + gr * row_stride + ch * 8);
-      r[i] = v;
-    }
+    for (int i = 0; i < N; i++)
+      r[i] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, i * RPP * (int)stride_bytes, 0));
   }
-  __device__ __forceinline__ void store(uint16_t* tile, int tid) const {
+  __device__ __forceinline__ void store(lds_ptr tile) const {
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-      const int id = tid + i * NT;
-      const int row = id / CH, ch = id % CH;
-      *reinterpret_cast<i32x4*>(tile + Tile<HD>::off(row, ch)) = r[i];
-    }
+    for (int i = 0; i < N; i++) *reinterpret_cast<MODA_LDS i32x4*>(tile + lds_off + i * RPP * HD) = r[i];
   }
 };
 
