@@ -117,22 +117,20 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
       const bool need_mask = !__all(full);
       MODA_LDS const float* lse_s = stat + cur * 2 * BM;
       MODA_LDS const float* del_s = lse_s + BM;
-      f32x16 s[2], dp[2];
+      // two 32-row halves of the query tile, one after the other: only one half's scores are live
 #pragma unroll
       for (int bb = 0; bb < 2; bb++) {
+        f32x16 s, dp;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          s[bb][i] = 0.f;
-          dp[bb][i] = 0.f;
+          s[i] = 0.f;
+          dp[i] = 0.f;
         }
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
-          s[bb] = mfma32<T>(lds_row_operand<HD>(Qs[cur], 32 * bb, kk, lane), Kr[kk], s[bb]);
-          dp[bb] = mfma32<T>(lds_row_operand<HD>(dOs[cur], 32 * bb, kk, lane), Vr[kk], dp[bb]);
+          s = mfma32<T>(lds_row_operand<HD>(Qs[cur], 32 * bb, kk, lane), Kr[kk], s);
+          dp = mfma32<T>(lds_row_operand<HD>(dOs[cur], 32 * bb, kk, lane), Vr[kk], dp);
         }
-      }
-#pragma unroll
-      for (int bb = 0; bb < 2; bb++)
 #pragma unroll
         for (int i4 = 0; i4 < 4; i4++) {
           const int row0 = 32 * bb + 8 * i4 + 4 * g;
@@ -141,28 +139,29 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
 #pragma unroll
           for (int j = 0; j < 4; j++) {
             const int i = 4 * i4 + j;
-            float p = fast_exp2(s[bb][i] * sc - lv[j]);
+            float p = fast_exp2(__builtin_fmaf(s[i], sc, -lv[j]));
             if (need_mask) {
               const int qr = q0 + row0 + j;
               p = (qr >= qlo && qr < qhi) ? p : 0.f;
             }
-            s[bb][i] = p;
-            dp[bb][i] = p * (dp[bb][i] - dl[j]);
+            s[i] = p;
+            dp[i] = p * (dp[i] - dl[j]);
           }
         }
-      i32x4 P[4], DS[4];
+        i32x4 P[2], DS[2];
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) {
-        P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
-        DS[ks] = pack8<T>(dp[ks >> 1], (ks & 1) * 8);
-      }
-#pragma unroll
-      for (int d = 0; d < DB; d++)
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-          dv[d] = mfma32<T>(lds_tr_operand<HD>(dOs[cur], 16 * ks, d, lane), P[ks], dv[d]);
-          dk[d] = mfma32<T>(lds_tr_operand<HD>(Qs[cur], 16 * ks, d, lane), DS[ks], dk[d]);
+        for (int ks = 0; ks < 2; ks++) {
+          P[ks] = pack8<T>(s, ks * 8);
+          DS[ks] = pack8<T>(dp, ks * 8);
         }
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+          for (int ks = 0; ks < 2; ks++) {
+            dv[d] = mfma32<T>(lds_tr_operand<HD>(dOs[cur], 32 * bb + 16 * ks, d, lane), P[ks], dv[d]);
+            dk[d] = mfma32<T>(lds_tr_operand<HD>(Qs[cur], 32 * bb + 16 * ks, d, lane), DS[ks], dk[d]);
+          }
+      }
     }
     if (it + 1 < niter) commit(cur ^ 1);
     __syncthreads();

@@ -71,17 +71,17 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
   const uint16_t* vdb = a.L > 0 ? a.vd + b * a.svd.b + hkv * a.svd.h : nullptr;
   const int TL = a.T * a.L;
 
-  TileLoader<HD, BN, 256> ldk, ldv;
-  ldk.init(tid);
-  ldv.init(tid);
+  AsyncTileLoader<HD, BN, 256> ld;
+  ld.init(tid);
   auto issue = [&](int it) {
+    const int st = it & 1;
     if (it < n_seq) {
-      ldk.load(kb, a.sk.t, it * BN, a.T, tid);
-      ldv.load(vb, a.sv.t, it * BN, a.T, tid);
+      ld.load(Ks[st], kb, a.sk.t, it * BN, a.T);
+      ld.load(Vs[st], vb, a.sv.t, it * BN, a.T);
     } else {
       const int c0 = dep0 + (it - n_seq) * BN;
-      ldk.load(kdb, a.skd.t, c0, TL, tid);
-      ldv.load(vdb, a.svd.t, c0, TL, tid);
+      ld.load(Ks[st], kdb, a.skd.t, c0, TL);
+      ld.load(Vs[st], vdb, a.svd.t, c0, TL);
     }
   };
 
@@ -93,11 +93,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
   float m = kNegInf, l = 0.f;
   const float sc = a.scale * kLog2e;
 
-  if (ntiles > 0) {
-    issue(0);
-    ldk.store(Ks[0]);
-    ldv.store(Vs[0]);
-  }
+  if (ntiles > 0) issue(0);
+  ld.wait_all();
   __syncthreads();
 
   for (int it = 0; it < ntiles; it++) {
@@ -174,10 +171,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
         for (int ks = 0; ks < 4; ks++) o[d] = mfma32<T>(lds_tr_operand<HD>(Vs[cur], 16 * ks, d, lane), P[ks], o[d]);
     }
 
-    if (it + 1 < ntiles) {
-      ldk.store(Ks[cur ^ 1]);
-      ldv.store(Vs[cur ^ 1]);
-    }
+    ld.wait_all();
     __syncthreads();
   }
 

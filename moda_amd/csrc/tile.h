@@ -177,6 +177,45 @@ struct TileLoader {
   }
 };
 
+// Global -> LDS staging without registers: gfx950 `buffer_load_dwordx4 ... lds`.
+// One wave-wide load fills 64 consecutive 16-byte LDS slots (lane l -> slot l);
+// the XOR swizzle is therefore applied on the GLOBAL side: the lane that owns
+// physical chunk p of a row fetches logical chunk p ^ swz(row).  Rows past the
+// end of the source are zero-filled by the buffer range check.  The loads are
+// asynchronous: call wait_all() before the barrier that publishes the tile.
+template <int HD, int ROWS, int NT>
+struct AsyncTileLoader {
+  static constexpr int CH = HD / 8;            // 16-byte chunks per row
+  static constexpr int NW = NT / 64;           // waves
+  static constexpr int RPW = 64 / CH;          // rows per wave-wide load
+  static constexpr int N = ROWS / (RPW * NW);  // loads per wave
+  static_assert(ROWS % (RPW * NW) == 0 && (RPW * NW) % 16 == 0, "tile must divide evenly");
+  int row_in_pass;  // row of this lane within one pass over the tile
+  int gchunk;       // logical chunk this lane fetches
+  int wave;
+
+  __device__ __forceinline__ void init(int tid) {
+    const int lane = tid & 63;
+    wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    row_in_pass = wave * RPW + lane / CH;
+    gchunk = (lane % CH) ^ Tile<HD>::swz(row_in_pass);
+  }
+  __device__ __forceinline__ void load(lds_ptr tile, const uint16_t* src, int64_t row_stride, int row0,
+                                       int row_end) const {
+    const int rows_left = row_end - row0;
+    const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
+    const uint32_t nbytes = rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(src + (int64_t)row0 * row_stride, nbytes);
+    const int voff = row_in_pass * (int)stride_bytes + gchunk * 16;
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(tile + (i * NW + wave) * 512), 16, voff,
+                                               i * NW * RPW * (int)stride_bytes, 0, 0);
+  }
+  // s_waitcnt vmcnt(0): every outstanding vector-memory load of this wave has landed
+  __device__ __forceinline__ static void wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+};
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
