@@ -2,29 +2,53 @@
 // (moda_v14.py:874-1248 and :1251-1454, moda_v16.py:1223-1425 and :1632-1834,
 // fda_v12.py:646-860, fla/ops/attn/parallel.py:299-440).
 //
-// A workgroup owns 128 key columns of one (batch, kv head) -- sequence keys or
-// flattened depth slots -- one column per lane pair, K and V rows held in
-// registers as MFMA B operands.  It streams 64-row query tiles (Q, dO, LSE,
-// delta) through LDS over exactly the query rows that can see its columns:
+// A workgroup (eight waves) owns 128 key columns of one (batch, kv head) --
+// sequence keys or flattened depth slots -- as four 32-column blocks, one column
+// per lane pair.  It streams 64-row query tiles (Q, dO, LSE, delta) through a
+// three-stage LDS ring over exactly the query rows that can see its columns:
 // all later tokens for a causal sequence key, the owner token's G rows (or the
-// rest of its chunk) for a depth slot.  All G folded rows, and in head-dim GQA
-// all G query heads, are reduced in registers, so every output row has one
-// writer and no atomics or partial buffers are needed.
+// rest of its chunk) for a depth slot.  Two waves share each column block and
+// split the work by ROLE so that each stays under 256 registers and the two
+// instruction streams overlap matrix and vector work on their SIMD:
+//   role A: S = Q K^T, P = exp2(S*c - lse), dV^T += dO^T P    (K in registers)
+//   role B: dP = dO V^T, dS = P (dP - delta), dK^T += Q^T dS  (V in registers)
+// P travels from A to B through a lane-private LDS mailbox in the 16-bit input
+// format; B runs one tile behind A, so one barrier per tile orders everything.
+// All G folded rows, and in head-dim GQA all G query heads, are reduced in
+// registers: every output row has one writer, no atomics, no partial buffers.
 #include "kargs.h"
 #include "tile.h"
 
 namespace moda {
 
+template <typename T>
+__device__ __forceinline__ void unpack2(int w, float& lo, float& hi);
+template <>
+__device__ __forceinline__ void unpack2<BF16>(int w, float& lo, float& hi) {
+  lo = __builtin_bit_cast(float, w << 16);
+  hi = __builtin_bit_cast(float, w & 0xffff0000);
+}
+template <>
+__device__ __forceinline__ void unpack2<FP16>(int w, float& lo, float& hi) {
+  const f16x2 v = __builtin_bit_cast(f16x2, w);
+  lo = (float)v[0];
+  hi = (float)v[1];
+}
+
 template <typename T, int HD>
-__global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
-  constexpr int BN = 128, BM = 64, KK = HD / 16, DB = HD / 32;
+__global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
+  constexpr int BN = 128, BM = 64, KK = HD / 16, DB = HD / 32, NST = 3;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
-  lds_ptr Qs[2] = {smem, smem + BM * HD};
-  lds_ptr dOs[2] = {smem + 2 * BM * HD, smem + 3 * BM * HD};
-  MODA_LDS float* stat = (MODA_LDS float*)(smem + 4 * BM * HD);  // [2][2][BM]: lse, delta per stage
+  // ring of NST stages, each: Q tile, dO tile; then the P mailbox; then lse/delta per stage
+  lds_ptr ring = smem;
+  MODA_LDS i32x4* mbox = (MODA_LDS i32x4*)(smem + NST * 2 * BM * HD);      // [2 parities][4 blocks][4][64 lanes]
+  MODA_LDS float* stat = (MODA_LDS float*)(mbox + 2 * 4 * 4 * 64);         // [NST][2][BM]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kblk = wave & 3;
+  const bool role_b = wave >= 4;
   const int BHk = a.B * a.Hkv;
   const int bh = blockIdx.x % BHk;
   const int ct = blockIdx.x / BHk;
@@ -33,18 +57,20 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
   const bool dep = ct >= n_seq_tiles;
   const int ncols = dep ? a.T * a.L : a.T;
   const int c_first = (dep ? ct - n_seq_tiles : ct) * BN;
-  const int c = c_first + wave * 32 + n;
+  const int c = c_first + kblk * 32 + n;
   const bool valid = c < ncols;
 
-  const uint16_t* ksrc = dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h;
-  const uint16_t* vsrc = dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h;
-  const int64_t kst = dep ? a.skd.t : a.sk.t, vst = dep ? a.svd.t : a.sv.t;
-  i32x4 Kr[KK], Vr[KK];
+  // stationary operand of this wave's role: K rows (A) or V rows (B)
+  i32x4 Sr[KK];
+  {
+    const uint16_t* src = role_b ? (dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h)
+                                 : (dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h);
+    const int64_t st = role_b ? (dep ? a.svd.t : a.sv.t) : (dep ? a.skd.t : a.sk.t);
 #pragma unroll
-  for (int kk = 0; kk < KK; kk++) {
-    i32x4 z = {0, 0, 0, 0};
-    Kr[kk] = valid ? *reinterpret_cast<const i32x4*>(ksrc + (int64_t)c * kst + 16 * kk + 8 * g) : z;
-    Vr[kk] = valid ? *reinterpret_cast<const i32x4*>(vsrc + (int64_t)c * vst + 16 * kk + 8 * g) : z;
+    for (int kk = 0; kk < KK; kk++) {
+      i32x4 z = {0, 0, 0, 0};
+      Sr[kk] = valid ? *reinterpret_cast<const i32x4*>(src + (int64_t)c * st + 16 * kk + 8 * g) : z;
+    }
   }
 
   // visible query-row interval of a column
@@ -67,129 +93,161 @@ __global__ __launch_bounds__(256) void dkv_kernel(const KArgs a) {
   const int nqt = (wg_hi + BM - 1) / BM - qt0;
   const int niter = nqt * a.hdiv;
 
-  TileLoader<HD, BM, 256> ldq, ldo;
-  ldq.init(tid);
-  ldo.init(tid);
-  float st_reg = 0.f;
+  AsyncTileLoader<HD, BM, 512> ld;
+  ld.init(tid);
   auto issue = [&](int it) {
     const int gh = it / nqt;
     const int q0 = (qt0 + it % nqt) * BM;
     const int hq = hkv * a.hdiv + gh;
-    ldq.load(a.q + b * a.sq.b + hq * a.sq.h, a.sq.t, q0, a.Tq, tid);
-    ldo.load(a.d_o + b * a.sdo.b + hq * a.sdo.h, a.sdo.t, q0, a.Tq, tid);
+    const int st = it % NST;
+    ld.load(ring + st * 2 * BM * HD, a.q + b * a.sq.b + hq * a.sq.h, a.sq.t, q0, a.Tq);
+    ld.load(ring + st * 2 * BM * HD + BM * HD, a.d_o + b * a.sdo.b + hq * a.sdo.h, a.sdo.t, q0, a.Tq);
     if (tid < 2 * BM) {
       const int row = q0 + (tid & (BM - 1));
-      st_reg = 0.f;
+      float v = 0.f;
       if (row < a.Tq)
-        st_reg = tid < BM ? a.lse[((int64_t)b * a.Tq + row) * a.Hq + hq]
-                          : a.delta[((int64_t)b * a.Hq + hq) * a.Tq + row];
+        v = tid < BM ? a.lse[((int64_t)b * a.Tq + row) * a.Hq + hq] : a.delta[((int64_t)b * a.Hq + hq) * a.Tq + row];
+      stat[st * 2 * BM + tid] = v;
     }
   };
-  auto commit = [&](int stage) {
-    ldq.store(Qs[stage]);
-    ldo.store(dOs[stage]);
-    if (tid < 2 * BM) stat[stage * 2 * BM + tid] = st_reg;
-  };
 
-  f32x16 dk[DB], dv[DB];
+  f32x16 acc[DB];  // dV^T (role A) or dK^T (role B)
 #pragma unroll
   for (int d = 0; d < DB; d++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      dk[d][i] = 0.f;
-      dv[d][i] = 0.f;
-    }
+    for (int i = 0; i < 16; i++) acc[d][i] = 0.f;
   const float sc = a.scale * kLog2e;
 
-  if (niter > 0) {
-    issue(0);
-    commit(0);
-  }
+  if (niter > 0) issue(0);
+  ld.wait_all();
   __syncthreads();
 
-  for (int it = 0; it < niter; it++) {
-    const int cur = it & 1;
+  // role A handles tile `it`, role B tile `it - 1`; one extra trip drains B
+  for (int it = 0; it <= niter; it++) {
     if (it + 1 < niter) issue(it + 1);
-    const int q0 = (qt0 + it % nqt) * BM;
-    const bool touches = (qhi > q0) && (qlo < q0 + BM) && (qhi > qlo);
-    if (__any(touches)) {
-      const bool full = (qlo <= q0) && (qhi >= q0 + BM);
-      const bool need_mask = !__all(full);
-      MODA_LDS const float* lse_s = stat + cur * 2 * BM;
-      MODA_LDS const float* del_s = lse_s + BM;
-      // two 32-row halves of the query tile, one after the other: only one half's scores are live
+    const int my = role_b ? it - 1 : it;
+    if (my >= 0 && my < niter) {
+      const int q0 = (qt0 + my % nqt) * BM;
+      const bool touches = (qhi > q0) && (qlo < q0 + BM) && (qhi > qlo);
+      if (__any(touches)) {
+        const int st = my % NST;
+        lds_cptr Qs = ring + st * 2 * BM * HD;
+        lds_cptr dOs = Qs + BM * HD;
+        MODA_LDS i32x4* mb = mbox + ((my & 1) * 4 + kblk) * 4 * 64 + lane;
+        if (!role_b) {
+          const bool full = (qlo <= q0) && (qhi >= q0 + BM);
+          const bool need_mask = !__all(full);
+          MODA_LDS const float* lse_s = stat + st * 2 * BM;
+          f32x16 s[2];
 #pragma unroll
-      for (int bb = 0; bb < 2; bb++) {
-        f32x16 s, dp;
+          for (int bb = 0; bb < 2; bb++) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          s[i] = 0.f;
-          dp[i] = 0.f;
-        }
+            for (int i = 0; i < 16; i++) s[bb][i] = 0.f;
 #pragma unroll
-        for (int kk = 0; kk < KK; kk++) {
-          s = mfma32<T>(lds_row_operand<HD>(Qs[cur], 32 * bb, kk, lane), Kr[kk], s);
-          dp = mfma32<T>(lds_row_operand<HD>(dOs[cur], 32 * bb, kk, lane), Vr[kk], dp);
-        }
+            for (int kk = 0; kk < KK; kk++)
+              s[bb] = mfma32<T>(lds_row_operand<HD>(Qs, 32 * bb, kk, lane), Sr[kk], s[bb]);
+          }
 #pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const int row0 = 32 * bb + 8 * i4 + 4 * g;
-          const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
-          const f32x4 dl = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + row0);
+          for (int bb = 0; bb < 2; bb++)
 #pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const int i = 4 * i4 + j;
-            float p = fast_exp2(__builtin_fmaf(s[i], sc, -lv[j]));
-            if (need_mask) {
-              const int qr = q0 + row0 + j;
-              p = (qr >= qlo && qr < qhi) ? p : 0.f;
+            for (int i4 = 0; i4 < 4; i4++) {
+              const int row0 = 32 * bb + 8 * i4 + 4 * g;
+              const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                const int i = 4 * i4 + j;
+                float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lv[j]));
+                if (need_mask) {
+                  const int qr = q0 + row0 + j;
+                  p = (qr >= qlo && qr < qhi) ? p : 0.f;
+                }
+                s[bb][i] = p;
+              }
             }
-            s[i] = p;
-            dp[i] = p * (dp[i] - dl[j]);
+          i32x4 P[4];
+#pragma unroll
+          for (int ks = 0; ks < 4; ks++) {
+            P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+            mb[ks * 64] = P[ks];
           }
-        }
-        i32x4 P[2], DS[2];
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-          P[ks] = pack8<T>(s, ks * 8);
-          DS[ks] = pack8<T>(dp, ks * 8);
-        }
+          for (int d = 0; d < DB; d++)
 #pragma unroll
-        for (int d = 0; d < DB; d++)
+            for (int ks = 0; ks < 4; ks++)
+              acc[d] = mfma32<T>(lds_tr_operand<HD>(dOs, 16 * ks, d, lane), P[ks], acc[d]);
+        } else {
+          MODA_LDS const float* del_s = stat + st * 2 * BM + BM;
+          f32x16 dp[2];
 #pragma unroll
-          for (int ks = 0; ks < 2; ks++) {
-            dv[d] = mfma32<T>(lds_tr_operand<HD>(dOs[cur], 32 * bb + 16 * ks, d, lane), P[ks], dv[d]);
-            dk[d] = mfma32<T>(lds_tr_operand<HD>(Qs[cur], 32 * bb + 16 * ks, d, lane), DS[ks], dk[d]);
+          for (int bb = 0; bb < 2; bb++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) dp[bb][i] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++)
+              dp[bb] = mfma32<T>(lds_row_operand<HD>(dOs, 32 * bb, kk, lane), Sr[kk], dp[bb]);
           }
+          i32x4 DS[4];
+#pragma unroll
+          for (int ks = 0; ks < 4; ks++) {
+            const int bb = ks >> 1;
+            const i32x4 pw = mb[ks * 64];
+            // accumulator registers 8*(ks&1) .. +7 of block bb: rows 32bb + 16(ks&1) + {0,8} + 4g + {0..3}
+            const int rbase = 32 * bb + 16 * (ks & 1) + 4 * g;
+            const f32x4 d0 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase);
+            const f32x4 d1 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase + 8);
+            float p[8];
+#pragma unroll
+            for (int w = 0; w < 4; w++) unpack2<T>(pw[w], p[2 * w], p[2 * w + 1]);
+            float ds[8];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              ds[j] = p[j] * (dp[bb][8 * (ks & 1) + j] - d0[j]);
+              ds[4 + j] = p[4 + j] * (dp[bb][8 * (ks & 1) + 4 + j] - d1[j]);
+            }
+            DS[ks][0] = pack2<T>(ds[0], ds[1]);
+            DS[ks][1] = pack2<T>(ds[2], ds[3]);
+            DS[ks][2] = pack2<T>(ds[4], ds[5]);
+            DS[ks][3] = pack2<T>(ds[6], ds[7]);
+          }
+#pragma unroll
+          for (int d = 0; d < DB; d++)
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++)
+              acc[d] = mfma32<T>(lds_tr_operand<HD>(Qs, 16 * ks, d, lane), DS[ks], acc[d]);
+        }
       }
     }
-    if (it + 1 < niter) commit(cur ^ 1);
+    ld.wait_all();
     __syncthreads();
   }
 
   if (valid) {
-    uint16_t* dkp = dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)c * a.sdkd.t
-                        : a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t;
-    uint16_t* dvp = dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)c * a.sdvd.t
-                        : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t;
+    uint16_t* outp;
+    float mul;
+    if (!role_b) {  // dV
+      outp = dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)c * a.sdvd.t
+                 : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t;
+      mul = 1.f;
+    } else {  // dK
+      outp = dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)c * a.sdkd.t
+                 : a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t;
+      mul = a.scale;
+    }
 #pragma unroll
     for (int d = 0; d < DB; d++)
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         i32x2 w;
-        w[0] = pack2<T>(dk[d][4 * i4 + 0] * a.scale, dk[d][4 * i4 + 1] * a.scale);
-        w[1] = pack2<T>(dk[d][4 * i4 + 2] * a.scale, dk[d][4 * i4 + 3] * a.scale);
-        *reinterpret_cast<i32x2*>(dkp + 32 * d + 8 * i4 + 4 * g) = w;
-        w[0] = pack2<T>(dv[d][4 * i4 + 0], dv[d][4 * i4 + 1]);
-        w[1] = pack2<T>(dv[d][4 * i4 + 2], dv[d][4 * i4 + 3]);
-        *reinterpret_cast<i32x2*>(dvp + 32 * d + 8 * i4 + 4 * g) = w;
+        w[0] = pack2<T>(acc[d][4 * i4 + 0] * mul, acc[d][4 * i4 + 1] * mul);
+        w[1] = pack2<T>(acc[d][4 * i4 + 2] * mul, acc[d][4 * i4 + 3] * mul);
+        *reinterpret_cast<i32x2*>(outp + 32 * d + 8 * i4 + 4 * g) = w;
       }
   }
 }
 
 template <typename T, int HD>
 hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = 4 * 64 * HD * sizeof(uint16_t) + 2 * 2 * 64 * sizeof(float);
+  constexpr size_t smem = 3 * 2 * 64 * HD * sizeof(uint16_t) + 2 * 4 * 4 * 64 * 16 + 3 * 2 * 64 * sizeof(float);
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dkv_kernel<T, HD>),
@@ -201,7 +259,7 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   const int64_t n_dep_tiles = a.L > 0 ? ((int64_t)a.T * a.L + 127) / 128 : 0;
   const int64_t nblk = (n_seq_tiles + n_dep_tiles) * a.B * a.Hkv;
   if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((dkv_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), smem, stream, a);
+  hipLaunchKernelGGL((dkv_kernel<T, HD>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
   return hipGetLastError();
 }
 
