@@ -16,6 +16,8 @@
 // format; B runs one tile behind A, so one barrier per tile orders everything.
 // All G folded rows, and in head-dim GQA all G query heads, are reduced in
 // registers: every output row has one writer, no atomics, no partial buffers.
+#include <type_traits>
+
 #include "kargs.h"
 #include "tile.h"
 
@@ -95,20 +97,31 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 
   AsyncTileLoader<HD, BM, 512> ld;
   ld.init(tid);
-  auto issue = [&](int it) {
-    const int gh = it / nqt;
-    const int q0 = (qt0 + it % nqt) * BM;
-    const int hq = hkv * a.hdiv + gh;
-    const int st = it % NST;
-    ld.load(ring + st * 2 * BM * HD, a.q + b * a.sq.b + hq * a.sq.h, a.sq.t, q0, a.Tq);
-    ld.load(ring + st * 2 * BM * HD + BM * HD, a.d_o + b * a.sdo.b + hq * a.sdo.h, a.sdo.t, q0, a.Tq);
-    if (tid < 2 * BM) {
-      const int row = q0 + (tid & (BM - 1));
-      float v = 0.f;
-      if (row < a.Tq)
-        v = tid < BM ? a.lse[((int64_t)b * a.Tq + row) * a.Hq + hq] : a.delta[((int64_t)b * a.Hq + hq) * a.Tq + row];
-      stat[st * 2 * BM + tid] = v;
+  // producer cursor: next tile to fetch = (query head ld_gh, query tile ld_qt) into ring stage ld_st
+  int ld_qt = 0, ld_gh = 0, ld_st = 0;
+  auto issue = [&]() {
+    const int q0 = (qt0 + ld_qt) * BM;
+    const int hq = hkv * a.hdiv + ld_gh;
+    lds_ptr stage = ring + ld_st * 2 * BM * HD;
+    ld.load(stage, a.q + b * a.sq.b + hq * a.sq.h, a.sq.t, q0, a.Tq);
+    ld.load(stage + BM * HD, a.d_o + b * a.sdo.b + hq * a.sdo.h, a.sdo.t, q0, a.Tq);
+    // per-row statistics straight into LDS as well: wave 0 fetches lse, wave 1 delta (one dword per lane)
+    const int rows = min(a.Tq - q0, BM);
+    if (wave == 0) {
+      const __amdgpu_buffer_rsrc_t rs =
+          make_rsrc(a.lse + ((int64_t)b * a.Tq + q0) * a.Hq + hq, rows > 0 ? ((rows - 1) * a.Hq + 1) * 4u : 0u);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(stat + ld_st * 2 * BM), 4, lane * a.Hq * 4, 0, 0,
+                                               0);
+    } else if (wave == 1) {
+      const __amdgpu_buffer_rsrc_t rs =
+          make_rsrc(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + q0, rows > 0 ? rows * 4u : 0u);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(stat + ld_st * 2 * BM + BM), 4, lane * 4, 0, 0, 0);
     }
+    if (++ld_qt == nqt) {
+      ld_qt = 0;
+      ld_gh++;
+    }
+    ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
   };
 
   f32x16 acc[DB];  // dV^T (role A) or dK^T (role B)
@@ -117,53 +130,60 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[d][i] = 0.f;
   const float sc = a.scale * kLog2e;
+  OperandAddr<HD> oa;
+  oa.init(lane);
 
-  if (niter > 0) issue(0);
+  if (niter > 0) issue();
   ld.wait_all();
   __syncthreads();
 
-  // role A handles tile `it`, role B tile `it - 1`; one extra trip drains B
+  // consumer cursor of this wave's role: query tile c_qt, ring stage c_st, mailbox parity c_par.
+  // Role A handles tile `it`, role B tile `it - 1`; one extra trip drains B.
+  int c_qt = 0, c_st = 0, c_par = 0;
   for (int it = 0; it <= niter; it++) {
-    if (it + 1 < niter) issue(it + 1);
-    const int my = role_b ? it - 1 : it;
-    if (my >= 0 && my < niter) {
-      const int q0 = (qt0 + my % nqt) * BM;
+    if (it + 1 < niter) issue();
+    const bool active = role_b ? (it >= 1) : (it < niter);
+    if (active) {
+      const int q0 = (qt0 + c_qt) * BM;
       const bool touches = (qhi > q0) && (qlo < q0 + BM) && (qhi > qlo);
       if (__any(touches)) {
-        const int st = my % NST;
-        lds_cptr Qs = ring + st * 2 * BM * HD;
+        lds_cptr Qs = ring + c_st * 2 * BM * HD;
         lds_cptr dOs = Qs + BM * HD;
-        MODA_LDS i32x4* mb = mbox + ((my & 1) * 4 + kblk) * 4 * 64 + lane;
+        MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * 4 * 64 + lane;
         if (!role_b) {
           const bool full = (qlo <= q0) && (qhi >= q0 + BM);
-          const bool need_mask = !__all(full);
-          MODA_LDS const float* lse_s = stat + st * 2 * BM;
+          MODA_LDS const float* lse_s = stat + c_st * 2 * BM;
           f32x16 s[2];
 #pragma unroll
           for (int bb = 0; bb < 2; bb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) s[bb][i] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < KK; kk++)
-              s[bb] = mfma32<T>(lds_row_operand<HD>(Qs, 32 * bb, kk, lane), Sr[kk], s[bb]);
+            for (int kk = 0; kk < KK; kk++) s[bb] = mfma32<T>(oa.row_operand(Qs, 32 * bb, kk), Sr[kk], s[bb]);
           }
+          auto probs = [&](auto masked) {
 #pragma unroll
-          for (int bb = 0; bb < 2; bb++)
+            for (int bb = 0; bb < 2; bb++)
 #pragma unroll
-            for (int i4 = 0; i4 < 4; i4++) {
-              const int row0 = 32 * bb + 8 * i4 + 4 * g;
-              const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
+              for (int i4 = 0; i4 < 4; i4++) {
+                const int row0 = 32 * bb + 8 * i4 + 4 * g;
+                const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
 #pragma unroll
-              for (int j = 0; j < 4; j++) {
-                const int i = 4 * i4 + j;
-                float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lv[j]));
-                if (need_mask) {
-                  const int qr = q0 + row0 + j;
-                  p = (qr >= qlo && qr < qhi) ? p : 0.f;
+                for (int j = 0; j < 4; j++) {
+                  const int i = 4 * i4 + j;
+                  float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lv[j]));
+                  if (decltype(masked)::value) {
+                    const int qr = q0 + row0 + j;
+                    p = (qr >= qlo && qr < qhi) ? p : 0.f;
+                  }
+                  s[bb][i] = p;
                 }
-                s[bb][i] = p;
               }
-            }
+          };
+          if (__all(full))
+            probs(std::false_type{});
+          else
+            probs(std::true_type{});
           i32x4 P[4];
 #pragma unroll
           for (int ks = 0; ks < 4; ks++) {
@@ -173,18 +193,16 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 #pragma unroll
           for (int d = 0; d < DB; d++)
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++)
-              acc[d] = mfma32<T>(lds_tr_operand<HD>(dOs, 16 * ks, d, lane), P[ks], acc[d]);
+            for (int ks = 0; ks < 4; ks++) acc[d] = mfma32<T>(oa.tr_operand(dOs, 16 * ks, d), P[ks], acc[d]);
         } else {
-          MODA_LDS const float* del_s = stat + st * 2 * BM + BM;
+          MODA_LDS const float* del_s = stat + c_st * 2 * BM + BM;
           f32x16 dp[2];
 #pragma unroll
           for (int bb = 0; bb < 2; bb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) dp[bb][i] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < KK; kk++)
-              dp[bb] = mfma32<T>(lds_row_operand<HD>(dOs, 32 * bb, kk, lane), Sr[kk], dp[bb]);
+            for (int kk = 0; kk < KK; kk++) dp[bb] = mfma32<T>(oa.row_operand(dOs, 32 * bb, kk), Sr[kk], dp[bb]);
           }
           i32x4 DS[4];
 #pragma unroll
@@ -212,10 +230,12 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 #pragma unroll
           for (int d = 0; d < DB; d++)
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++)
-              acc[d] = mfma32<T>(lds_tr_operand<HD>(Qs, 16 * ks, d, lane), DS[ks], acc[d]);
+            for (int ks = 0; ks < 4; ks++) acc[d] = mfma32<T>(oa.tr_operand(Qs, 16 * ks, d), DS[ks], acc[d]);
         }
       }
+      if (++c_qt == nqt) c_qt = 0;
+      c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+      c_par ^= 1;
     }
     ld.wait_all();
     __syncthreads();

@@ -117,6 +117,8 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) dq[d][i] = 0.f;
   const float sc = a.scale * kLog2e;
+  OperandAddr<HD> oa;
+  oa.init(lane);
 
   if (ntiles > 0) issue(0);
   ld.wait_all();
@@ -144,8 +146,8 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
         }
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
-          s[bb] = mfma32<T>(lds_row_operand<HD>(Ks[cur], 32 * bb, kk, lane), Qr[kk], s[bb]);
-          dp[bb] = mfma32<T>(lds_row_operand<HD>(Vs[cur], 32 * bb, kk, lane), dOr[kk], dp[bb]);
+          s[bb] = mfma32<T>(oa.row_operand(Ks[cur], 32 * bb, kk), Qr[kk], s[bb]);
+          dp[bb] = mfma32<T>(oa.row_operand(Vs[cur], 32 * bb, kk), dOr[kk], dp[bb]);
         }
       }
 #pragma unroll
@@ -166,7 +168,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
       for (int d = 0; d < DB; d++)
 #pragma unroll
         for (int ks = 0; ks < 4; ks++)
-          dq[d] = mfma32<T>(lds_tr_operand<HD>(Ks[cur], 16 * ks, d, lane), DS[ks], dq[d]);
+          dq[d] = mfma32<T>(oa.tr_operand(Ks[cur], 16 * ks, d), DS[ks], dq[d]);
     }
 
     ld.wait_all();

@@ -92,6 +92,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
     for (int i = 0; i < 16; i++) o[d][i] = 0.f;
   float m = kNegInf, l = 0.f;
   const float sc = a.scale * kLog2e;
+  OperandAddr<HD> oa;
+  oa.init(lane);
 
   if (ntiles > 0) issue(0);
   ld.wait_all();
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
         for (int i = 0; i < 16; i++) s[bb][i] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < KK; kk++)
-          s[bb] = mfma32<T>(lds_row_operand<HD>(Ks[cur], 32 * bb, kk, lane), Qr[kk], s[bb]);
+          s[bb] = mfma32<T>(oa.row_operand(Ks[cur], 32 * bb, kk), Qr[kk], s[bb]);
       }
       // row maximum of the raw scores (scale > 0, so it commutes with the max)
       float mx = kNegInf;
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
 #pragma unroll
       for (int d = 0; d < DB; d++)
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) o[d] = mfma32<T>(lds_tr_operand<HD>(Vs[cur], 16 * ks, d, lane), P[ks], o[d]);
+        for (int ks = 0; ks < 4; ks++) o[d] = mfma32<T>(oa.tr_operand(Vs[cur], 16 * ks, d), P[ks], o[d]);
     }
 
     ld.wait_all();

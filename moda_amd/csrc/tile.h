@@ -103,15 +103,13 @@ struct Tile {
   __device__ __forceinline__ static int off(int row, int chunk) { return row * HD + ((chunk ^ swz(row)) << 3); }
 };
 
-// Row operand: lane (n, g) gets elements [16*kk + 8g, +8) of row (row0 + n).
+// Per-lane LDS offsets of the two operand read patterns, computed once.  Tile
+// rows are only ever offset by multiples of 16, which leaves the swizzle of a
+// lane's row unchanged, so every read is `tile + precomputed + compile-time constant`.
+//
+// Row operand: lane (n, g) gets elements [16*kk + 8g, +8) of tile row (row0 + n).
 // Serves as MFMA A (M = tile rows) or B (N = tile rows) with K = head dim.
-template <int HD>
-__device__ __forceinline__ i32x4 lds_row_operand(lds_cptr tile, int row0, int kk, int lane) {
-  const int n = lane & 31, g = lane >> 5;
-  lds_cptr p = tile + Tile<HD>::off(row0 + n, 2 * kk + g);
-  return *reinterpret_cast<MODA_LDS const i32x4*>(p);
-}
-
+//
 // Transposed operand: lane (n, g) gets, for head-dim column d = 32*dblk + n,
 // tile rows rb + 4g + {0,1,2,3} (k slots 0..3) and rb + 8 + 4g + {0,1,2,3}
 // (k slots 4..7) -- exactly the rows that accumulator registers 8s..8s+7 of a
@@ -120,24 +118,42 @@ __device__ __forceinline__ i32x4 lds_row_operand(lds_cptr tile, int row0, int kk
 // r supplies the address of 4 consecutive elements; result lane i receives
 // element (i & 3) of source lanes 4j + (i >> 2), j = 0..3.
 template <int HD>
-__device__ __forceinline__ i32x4 lds_tr_operand(lds_cptr tile, int rb, int dblk, int lane) {
-  const int g = lane >> 5;
-  const int r16 = lane & 15;
-  const int row = rb + 4 * g + (r16 >> 2);
-  const int dcol = 32 * dblk + ((lane >> 4) & 1) * 16 + (r16 & 3) * 4;
-  lds_cptr p0 = tile + Tile<HD>::off(row, dcol >> 3) + (dcol & 7);
-  lds_cptr p1 = tile + Tile<HD>::off(row + 8, dcol >> 3) + (dcol & 7);
-  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(p0));
-  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(p1));
-  i32x2 l2 = __builtin_bit_cast(i32x2, lo);
-  i32x2 h2 = __builtin_bit_cast(i32x2, hi);
-  i32x4 r;
-  r[0] = l2[0];
-  r[1] = l2[1];
-  r[2] = h2[0];
-  r[3] = h2[1];
-  return r;
-}
+struct OperandAddr {
+  static constexpr int KK = HD / 16, DB = HD / 32;
+  int row[KK];
+  int tr[2][DB];
+
+  __device__ __forceinline__ void init(int lane) {
+    const int n = lane & 31, g = lane >> 5, r16 = lane & 15;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) row[kk] = Tile<HD>::off(n, 2 * kk + g);
+#pragma unroll
+    for (int hi = 0; hi < 2; hi++)
+#pragma unroll
+      for (int d = 0; d < DB; d++) {
+        const int r = 4 * g + (r16 >> 2) + 8 * hi;
+        const int dcol = 32 * d + ((lane >> 4) & 1) * 16 + (r16 & 3) * 4;
+        tr[hi][d] = Tile<HD>::off(r, dcol >> 3) + (dcol & 7);
+      }
+  }
+  // row0 must be a multiple of 16
+  __device__ __forceinline__ i32x4 row_operand(lds_cptr tile, int row0, int kk) const {
+    return *reinterpret_cast<MODA_LDS const i32x4*>(tile + row[kk] + row0 * HD);
+  }
+  // rb must be a multiple of 16
+  __device__ __forceinline__ i32x4 tr_operand(lds_cptr tile, int rb, int dblk) const {
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(tile + tr[0][dblk] + rb * HD));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MODA_LDS s16x4*)(tile + tr[1][dblk] + rb * HD));
+    i32x2 l2 = __builtin_bit_cast(i32x2, lo);
+    i32x2 h2 = __builtin_bit_cast(i32x2, hi);
+    i32x4 r;
+    r[0] = l2[0];
+    r[1] = l2[1];
+    r[2] = h2[0];
+    r[3] = h2[1];
+    return r;
+  }
+};
 
 // Raw buffer resource over `nbytes` bytes at `base` (wave-uniform): loads past the end return zero.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t nbytes) {
