@@ -112,14 +112,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
       const bool full = (lo <= col0) && (hi >= col0 + BN);
       const bool need_mask = !__all(full);
       f32x16 s[2];
-#pragma unroll
-      for (int bb = 0; bb < 2; bb++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) s[bb][i] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < KK; kk++)
-          s[bb] = mfma32<T>(oa.row_operand(Ks[cur], 32 * bb, kk), Qr[kk], s[bb]);
-      }
+      mfma_rows<T, HD, 2, 4>(oa, Ks[cur], Qr, s);
+      // first V^T operands start travelling while the softmax runs
+      TrPipe<T, HD, 4, 4> pv;
+      pv.prefetch(oa, Vs[cur]);
       // row maximum of the raw scores (scale > 0, so it commutes with the max)
       float mx = kNegInf;
       if (need_mask) {
@@ -128,9 +124,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
 #pragma unroll
           for (int i = 0; i < 16; i++) {
             const int c = col0 + 32 * bb + acc_row(i, g);
-            const float x = (c >= lo && c < hi) ? s[bb][i] : kNegInf;
-            s[bb][i] = x;
-            mx = fmaxf(mx, x);
+            mx = fmaxf(mx, (c >= lo && c < hi) ? s[bb][i] : kNegInf);
           }
       } else {
 #pragma unroll
@@ -154,23 +148,32 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
       }
       const float neg_m = (m == kNegInf) ? 0.f : -m;
       float rs = 0.f;
-#pragma unroll
-      for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m));
-          s[bb][i] = p;
-          rs += p;
-        }
-      rs += xor32(rs);
-      l += rs;
       i32x4 P[4];
+      if (need_mask) {
+#pragma unroll
+        for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const int c = col0 + 32 * bb + acc_row(i, g);
+            const float p = (c >= lo && c < hi) ? fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m)) : 0.f;
+            s[bb][i] = p;
+            rs += p;
+          }
+      } else {
+#pragma unroll
+        for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m));
+            s[bb][i] = p;
+            rs += p;
+          }
+      }
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
-#pragma unroll
-      for (int d = 0; d < DB; d++)
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) o[d] = mfma32<T>(oa.tr_operand(Vs[cur], 16 * ks, d), P[ks], o[d]);
+      rs += xor32(rs);
+      l += rs;
+      pv.run(oa, Vs[cur], P, o);
     }
 
     ld.wait_all();

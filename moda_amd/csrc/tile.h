@@ -155,6 +155,91 @@ struct OperandAddr {
   }
 };
 
+// Software-pipelined MFMA sequences.  The compiler, left alone, issues each LDS
+// operand read immediately before the MFMA that consumes it and so exposes the
+// full LDS latency once per MFMA; these helpers keep DEPTH operand reads in
+// flight ahead of the matrix pipe and pin that order with scheduling barriers.
+// Consecutive MFMAs always target different accumulators.
+
+// acc[bb] = sum_kk rows(tile, 32*bb + n, kk) x breg[kk]   (accumulators start at zero)
+template <typename T, int HD, int NB, int DEPTH>
+__device__ __forceinline__ void mfma_rows(const OperandAddr<HD>& oa, lds_cptr tile, const i32x4 (&breg)[HD / 16],
+                                          f32x16 (&acc)[NB]) {
+  constexpr int KK = HD / 16, N = NB * KK;
+  i32x4 ops[N];
+#pragma unroll
+  for (int j = 0; j < DEPTH && j < N; j++) ops[j] = oa.row_operand(tile, 32 * (j % NB), j / NB);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < N; j++) {
+    if (j + DEPTH < N) ops[j + DEPTH] = oa.row_operand(tile, 32 * ((j + DEPTH) % NB), (j + DEPTH) / NB);
+    const int bb = j % NB, kk = j / NB;
+    if (kk == 0) {
+      f32x16 z;
+#pragma unroll
+      for (int i = 0; i < 16; i++) z[i] = 0.f;
+      acc[bb] = mfma32<T>(ops[j], breg[kk], z);
+    } else {
+      acc[bb] = mfma32<T>(ops[j], breg[kk], acc[bb]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// Two tiles against two register operands in one pipeline:
+// acc0[bb] = rows(tile0) x breg0, acc1[bb] = rows(tile1) x breg1.
+template <typename T, int HD, int NB, int DEPTH>
+__device__ __forceinline__ void mfma_rows2(const OperandAddr<HD>& oa, lds_cptr tile0, const i32x4 (&breg0)[HD / 16],
+                                           f32x16 (&acc0)[NB], lds_cptr tile1, const i32x4 (&breg1)[HD / 16],
+                                           f32x16 (&acc1)[NB]) {
+  constexpr int KK = HD / 16, N = 2 * NB * KK;
+  i32x4 ops[N];
+  // step j: which = j & 1, bb = (j >> 1) % NB, kk = (j >> 1) / NB
+#pragma unroll
+  for (int j = 0; j < DEPTH && j < N; j++)
+    ops[j] = oa.row_operand((j & 1) ? tile1 : tile0, 32 * ((j >> 1) % NB), (j >> 1) / NB);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < N; j++) {
+    if (j + DEPTH < N) {
+      const int jn = j + DEPTH;
+      ops[jn] = oa.row_operand((jn & 1) ? tile1 : tile0, 32 * ((jn >> 1) % NB), (jn >> 1) / NB);
+    }
+    const int bb = (j >> 1) % NB, kk = (j >> 1) / NB;
+    f32x16 z;
+#pragma unroll
+    for (int i = 0; i < 16; i++) z[i] = 0.f;
+    if (j & 1)
+      acc1[bb] = mfma32<T>(ops[j], breg1[kk], kk == 0 ? z : acc1[bb]);
+    else
+      acc0[bb] = mfma32<T>(ops[j], breg0[kk], kk == 0 ? z : acc0[bb]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// acc[d] += tr(tile, 16*ks, d) x breg[ks]  for ks < NKS, d < HD/32.  prefetch() may be
+// called early (before the code that produces breg) to have the first operands waiting.
+template <typename T, int HD, int NKS, int DEPTH>
+struct TrPipe {
+  static constexpr int DB = HD / 32, N = NKS * DB;
+  i32x4 ops[N];
+  __device__ __forceinline__ void prefetch(const OperandAddr<HD>& oa, lds_cptr tile) {
+#pragma unroll
+    for (int j = 0; j < DEPTH && j < N; j++) ops[j] = oa.tr_operand(tile, 16 * (j / DB), j % DB);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __device__ __forceinline__ void run(const OperandAddr<HD>& oa, lds_cptr tile, const i32x4 (&breg)[NKS],
+                                      f32x16 (&acc)[DB]) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+      if (j + DEPTH < N) ops[j + DEPTH] = oa.tr_operand(tile, 16 * ((j + DEPTH) / DB), (j + DEPTH) % DB);
+      acc[j % DB] = mfma32<T>(ops[j], breg[j / DB], acc[j % DB]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+};
+
 // Raw buffer resource over `nbytes` bytes at `base` (wave-uniform): loads past the end return zero.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t nbytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)nbytes, 0x00020000);
