@@ -126,6 +126,31 @@ def cpu_baseline(B, T, Hkv, G, D, L, mode, cb, target_seconds=15.0):
     }
 
 
+def bench_reorg(dev, B, T, Hkv, D, L, iters=10):
+    """Depth-KV reorganisation kernel at the workload's shape: L per-layer [B,T,Hkv,D] bf16 tensors ->
+    token-major cache [B,T*L,Hkv,D] (one tensor; K and V each cost this).  HBM-bound: algorithmic bytes =
+    read + write of B*T*L*Hkv*D*2."""
+    import torch
+
+    from moda_amd import depth_cache
+
+    layers = [torch.randn(B, T, Hkv, D, device=dev).bfloat16() for _ in range(L)]
+    cache = torch.empty(B, T * L, Hkv, D, dtype=torch.bfloat16, device=dev)
+    for _ in range(2):
+        depth_cache._reorg_fwd(layers, cache, 0, L)
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        depth_cache._reorg_fwd(layers, cache, 0, L)
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / iters
+    nbytes = 2 * B * T * L * Hkv * D * 2
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"kernel": "reorg_kernel", "ms": ms, "bytes": nbytes, "achieved": gbs, "unit": "GB/s",
+            "peak": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS, "bound": "hbm"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -252,6 +277,8 @@ def main():
         tw_value = 3.5 * tw["flops_fwd"] / (tw["ms_step"] * 1e-3) / 1e12
         out["plain_causal_twin"] = {"tflops": tw_value, "ms_per_step": tw["ms_step"],
                                     "moda_over_twin": value / tw_value}
+    if L > 0:
+        out["depth_reorg"] = bench_reorg(dev, B, T, Hkv, D, L)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, T, Hkv, G, D, L, mode, cb)
     print(json.dumps(out))

@@ -9,6 +9,7 @@
 // dQ^T += K^T * dS^T, K^T coming from the LDS transpose read of the K tile.
 #include "kargs.h"
 #include "tile.h"
+#include "tuning.h"
 
 namespace moda {
 
@@ -36,17 +37,18 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a) {
 }
 
 template <typename T, int HD>
-__global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
-  constexpr int BM = 128, BN = 64, KK = HD / 16, DB = HD / 32;
+__global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const KArgs a) {
+  constexpr int BM = kRowBM, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * kRowWaves, NST = kRowStages, DIST = kRowDist;
+  static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
-  lds_ptr Ks[2] = {smem, smem + BN * HD};
-  lds_ptr Vs[2] = {smem + 2 * BN * HD, smem + 3 * BN * HD};
+  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
   const int BH = a.B * a.Hq;
   const int bh = blockIdx.x % BH;
-  const int qt = a.nqt - 1 - blockIdx.x / BH;
+  const int nqt = (a.Tq + BM - 1) / BM;
+  const int qt = nqt - 1 - blockIdx.x / BH;
   const int b = bh / a.Hq, hq = bh % a.Hq, hkv = hq / a.hdiv;
   const int r = qt * BM + wave * 32 + n;
   const bool valid = r < a.Tq;
@@ -97,18 +99,29 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
   const uint16_t* vdb = a.L > 0 ? a.vd + b * a.svd.b + hkv * a.svd.h : nullptr;
   const int TL = a.T * a.L;
 
-  AsyncTileLoader<HD, BN, 256> ld;
+  typedef AsyncTileLoader<HD, BN, NT> Loader;
+  constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
+  Loader ld;
   ld.init(tid);
+  int ld_st = 0;  // ring stage the next issued tile goes to
   auto issue = [&](int it) {
-    const int st = it & 1;
+    lds_ptr Kt = smem + ld_st * 2 * BN * HD;
     if (it < n_seq) {
-      ld.load(Ks[st], kb, a.sk.t, it * BN, a.T);
-      ld.load(Vs[st], vb, a.sv.t, it * BN, a.T);
+      ld.load(Kt, kb, a.sk.t, it * BN, a.T);
+      ld.load(Kt + BN * HD, vb, a.sv.t, it * BN, a.T);
     } else {
       const int c0 = dep0 + (it - n_seq) * BN;
-      ld.load(Ks[st], kdb, a.skd.t, c0, TL);
-      ld.load(Vs[st], vdb, a.svd.t, c0, TL);
+      ld.load(Kt, kdb, a.skd.t, c0, TL);
+      ld.load(Kt + BN * HD, vdb, a.svd.t, c0, TL);
     }
+    ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
+  };
+  // wait until tile `next` has landed; tiles next+1 .. next+DIST-1 may still be in flight
+  auto wait_tile = [&](int next) {
+    if (DIST == 2 && next + 1 < ntiles)
+      Loader::template wait_but<LPT>();
+    else
+      Loader::wait_all();
   };
 
   f32x16 dq[DB];
@@ -120,13 +133,17 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
   OperandAddr<HD> oa;
   oa.init(lane);
 
-  if (ntiles > 0) issue(0);
-  ld.wait_all();
+#pragma unroll
+  for (int j = 0; j < DIST; j++)
+    if (j < ntiles) issue(j);
+  wait_tile(0);
   __syncthreads();
+  int c_st = 0;  // ring stage of the tile being consumed
 
   for (int it = 0; it < ntiles; it++) {
-    const int cur = it & 1;
-    if (it + 1 < ntiles) issue(it + 1);
+    if (it + DIST < ntiles) issue(it + DIST);
+    lds_cptr Kc = smem + c_st * 2 * BN * HD;
+    lds_cptr Vc = Kc + BN * HD;
 
     const bool dep = it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
@@ -146,8 +163,8 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
         }
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
-          s[bb] = mfma32<T>(oa.row_operand(Ks[cur], 32 * bb, kk), Qr[kk], s[bb]);
-          dp[bb] = mfma32<T>(oa.row_operand(Vs[cur], 32 * bb, kk), dOr[kk], dp[bb]);
+          s[bb] = mfma32<T>(oa.row_operand(Kc, 32 * bb, kk), Qr[kk], s[bb]);
+          dp[bb] = mfma32<T>(oa.row_operand(Vc, 32 * bb, kk), dOr[kk], dp[bb]);
         }
       }
 #pragma unroll
@@ -168,10 +185,11 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const KArgs a) {
       for (int d = 0; d < DB; d++)
 #pragma unroll
         for (int ks = 0; ks < 4; ks++)
-          dq[d] = mfma32<T>(oa.tr_operand(Ks[cur], 16 * ks, d), DS[ks], dq[d]);
+          dq[d] = mfma32<T>(oa.tr_operand(Kc, 16 * ks, d), DS[ks], dq[d]);
     }
 
-    ld.wait_all();
+    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    wait_tile(it + 1);
     __syncthreads();
   }
 
@@ -199,7 +217,7 @@ hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
 
 template <typename T, int HD>
 hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = 4 * 64 * HD * sizeof(uint16_t);
+  constexpr size_t smem = (size_t)kRowStages * 2 * 64 * HD * sizeof(uint16_t);
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<T, HD>),
@@ -207,9 +225,9 @@ hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  const int64_t nblk = (int64_t)a.nqt * a.B * a.Hq;
+  const int64_t nblk = (int64_t)((a.Tq + kRowBM - 1) / kRowBM) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((dq_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), smem, stream, a);
+  hipLaunchKernelGGL((dq_kernel<T, HD>), dim3((unsigned)nblk), dim3(64 * kRowWaves), smem, stream, a);
   return hipGetLastError();
 }
 

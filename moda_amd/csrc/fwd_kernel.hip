@@ -2,30 +2,39 @@
 // query's depth-KV slots (the computation of moda_v14.py:45-378,
 // moda_v16.py:39-352, fda_v12.py:44-253 and fla/ops/attn/parallel.py:18-143).
 //
-// Work split: one workgroup = 128 query rows of one (batch, query head), four
-// 64-lane waves of 32 rows each.  Scores are produced transposed,
-// S^T = K * Q^T, so each lane owns ONE query row: row statistics need a single
-// cross-lane exchange and P^T is already laid out as the B operand of
-// O^T += V^T * P^T.  K and V tiles (64 columns) are staged through LDS, V is
-// read with the LDS transpose load.  Depth columns are extra column tiles with
-// a different per-row visible interval.
+// Work split: one workgroup = 32 query rows per wave of one (batch, query
+// head).  Scores are produced transposed, S^T = K * Q^T, so each lane owns ONE
+// query row: row statistics need a single half-wave exchange and P^T is already
+// laid out as the B operand of O^T += V^T * P^T.  K and V tiles (64 columns)
+// travel global -> LDS without touching registers, a ring of stages keeps the
+// loads ahead of the math, V is read with the LDS transpose load.  Depth
+// columns are extra column tiles with a different per-row visible interval.
+//
+// Vector-ALU instructions do not overlap with MFMA on this hardware, so the
+// loop over column tiles is split in two: tiles every row of the workgroup sees
+// completely run a body without any masking or visibility tests; boundary and
+// depth tiles run the masked body.
+#include <type_traits>
+
 #include "kargs.h"
 #include "tile.h"
+#include "tuning.h"
 
 namespace moda {
 
 template <typename T, int HD>
-__global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
-  constexpr int BM = 128, BN = 64, KK = HD / 16, DB = HD / 32;
+__global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void fwd_kernel(const KArgs a) {
+  constexpr int BM = kRowBM, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * kRowWaves, NST = kRowStages,
+                DIST = kRowDist;
+  static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  lds_ptr smem = (lds_ptr)smem_raw;
-  lds_ptr Ks[2] = {smem, smem + BN * HD};
-  lds_ptr Vs[2] = {smem + 2 * BN * HD, smem + 3 * BN * HD};
+  lds_ptr smem = (lds_ptr)smem_raw;  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
   const int BH = a.B * a.Hq;
   const int bh = blockIdx.x % BH;
-  const int qt = a.nqt - 1 - blockIdx.x / BH;  // heavy (late) tiles first
+  const int nqt = (a.Tq + BM - 1) / BM;
+  const int qt = nqt - 1 - blockIdx.x / BH;  // heavy (late) tiles first
   const int b = bh / a.Hq, hq = bh % a.Hq, hkv = hq / a.hdiv;
   const int r = qt * BM + wave * 32 + n;
   const bool valid = r < a.Tq;
@@ -55,8 +64,13 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
   const int r_first = qt * BM;
   const int r_last = min(a.Tq, r_first + BM) - 1;
   const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
-  int n_seq = 0;
-  if (a.has_seq) n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
+  int n_seq = 0, n_full = 0;
+  if (a.has_seq) {
+    n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
+    // leading sequence tiles that every row of the workgroup sees completely (padding rows of the
+    // last workgroup compute on zero queries there and are never stored)
+    n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
+  }
   int dep0 = 0, n_dep = 0;
   if (a.L > 0) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
@@ -65,24 +79,35 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
   }
   const int ntiles = n_seq + n_dep;
 
-  const uint16_t* kb = a.has_seq ? a.k + b * a.sk.b + hkv * a.sk.h : nullptr;
-  const uint16_t* vb = a.has_seq ? a.v + b * a.sv.b + hkv * a.sv.h : nullptr;
-  const uint16_t* kdb = a.L > 0 ? a.kd + b * a.skd.b + hkv * a.skd.h : nullptr;
-  const uint16_t* vdb = a.L > 0 ? a.vd + b * a.svd.b + hkv * a.svd.h : nullptr;
-  const int TL = a.T * a.L;
-
-  AsyncTileLoader<HD, BN, 256> ld;
+  typedef AsyncTileLoader<HD, BN, NT> Loader;
+  constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
+  Loader ld;
   ld.init(tid);
+  // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
+  // producer reaches the first depth tile
+  typename Loader::Source srcK, srcV;
+  if (a.has_seq && n_seq > 0) {
+    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
+    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
+  }
+  int ld_st = 0;  // ring stage the next issued tile goes to
   auto issue = [&](int it) {
-    const int st = it & 1;
-    if (it < n_seq) {
-      ld.load(Ks[st], kb, a.sk.t, it * BN, a.T);
-      ld.load(Vs[st], vb, a.sv.t, it * BN, a.T);
-    } else {
-      const int c0 = dep0 + (it - n_seq) * BN;
-      ld.load(Ks[st], kdb, a.skd.t, c0, TL);
-      ld.load(Vs[st], vdb, a.svd.t, c0, TL);
+    lds_ptr Kt = smem + ld_st * 2 * BN * HD;
+    if (it == n_seq) {
+      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
+      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
+    const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
+    ld.load_from(Kt, srcK, row0);
+    ld.load_from(Kt + BN * HD, srcV, row0);
+    ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
+  };
+  // wait until tile `next` has landed; tiles next+1 .. next+DIST-1 may still be in flight
+  auto wait_tile = [&](int next) {
+    if (DIST == 2 && next + 1 < ntiles)
+      Loader::template wait_but<LPT>();
+    else
+      Loader::wait_all();
   };
 
   f32x16 o[DB];
@@ -95,88 +120,95 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
   OperandAddr<HD> oa;
   oa.init(lane);
 
-  if (ntiles > 0) issue(0);
-  ld.wait_all();
+#pragma unroll
+  for (int j = 0; j < DIST; j++)
+    if (j < ntiles) issue(j);
+  wait_tile(0);
   __syncthreads();
+  int c_st = 0;  // ring stage of the tile being consumed
 
-  for (int it = 0; it < ntiles; it++) {
-    const int cur = it & 1;
-    if (it + 1 < ntiles) issue(it + 1);
+  // one column tile: S^T = K Q^T, online softmax, O^T += V^T P^T
+  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, int lo, int hi) {
+    constexpr bool MASKED = decltype(masked)::value;
+    f32x16 s[2];
+    mfma_rows<T, HD, 2, 4>(oa, Kc, Qr, s);
+    // first V^T operands start travelling while the softmax runs
+    TrPipe<T, HD, 4, 2> pv;
+    pv.prefetch(oa, Vc);
+    // row maximum of the raw scores (scale > 0, so it commutes with the max)
+    float mx = kNegInf;
+#pragma unroll
+    for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        if (MASKED) {
+          const int c = col0 + 32 * bb + acc_row(i, g);
+          mx = fmaxf(mx, (c >= lo && c < hi) ? s[bb][i] : kNegInf);
+        } else {
+          mx = fmaxf(mx, s[bb][i]);
+        }
+      }
+    mx = pair_max(mx) * sc;
+    // The exponent reference m only moves when some row's maximum outgrows it by more than 2^8:
+    // p stays <= 256, exact in fp32 accumulation and harmless in the 16-bit P, and the
+    // rescale of O is skipped on almost every tile.
+    if (__any(mx > m + 8.f)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = fast_exp2(m - ((m_new == kNegInf) ? 0.f : m_new));
+      l *= alpha;
+      m = m_new;
+#pragma unroll
+      for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[d][i] *= alpha;
+    }
+    const float neg_m = (m == kNegInf) ? 0.f : -m;
+    float rs0 = 0.f, rs1 = 0.f;  // fp32 row sum of the unrounded probabilities, as the reference keeps it
+#pragma unroll
+    for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m));
+        if (MASKED) {
+          const int c = col0 + 32 * bb + acc_row(i, g);
+          p = (c >= lo && c < hi) ? p : 0.f;
+        }
+        s[bb][i] = p;
+        if (i & 1)
+          rs1 += p;
+        else
+          rs0 += p;
+      }
+    i32x4 P[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+    l += pair_sum(rs0 + rs1);
+    pv.run(oa, Vc, P, o);
+  };
 
+  // phase 1: tiles fully visible to every row -- no masks, no visibility tests
+  for (int it = 0; it < n_full; it++) {
+    if (it + DIST < ntiles) issue(it + DIST);
+    lds_cptr Kc = smem + c_st * 2 * BN * HD;
+    tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, 0, 0);
+    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    wait_tile(it + 1);
+    __syncthreads();
+  }
+  // phase 2: boundary sequence tiles and depth tiles
+  for (int it = n_full; it < ntiles; it++) {
+    if (it + DIST < ntiles) issue(it + DIST);
     const bool dep = it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
     const int lo = dep ? dlo : 0;
     const int hi = dep ? dhi : shi;
     const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
     if (__any(touches)) {
-      const bool full = (lo <= col0) && (hi >= col0 + BN);
-      const bool need_mask = !__all(full);
-      f32x16 s[2];
-      mfma_rows<T, HD, 2, 4>(oa, Ks[cur], Qr, s);
-      // first V^T operands start travelling while the softmax runs
-      TrPipe<T, HD, 4, 4> pv;
-      pv.prefetch(oa, Vs[cur]);
-      // row maximum of the raw scores (scale > 0, so it commutes with the max)
-      float mx = kNegInf;
-      if (need_mask) {
-#pragma unroll
-        for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int c = col0 + 32 * bb + acc_row(i, g);
-            mx = fmaxf(mx, (c >= lo && c < hi) ? s[bb][i] : kNegInf);
-          }
-      } else {
-#pragma unroll
-        for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[bb][i]);
-      }
-      mx = fmaxf(mx, xor32(mx)) * sc;
-      // The exponent reference m only moves when some row's maximum outgrows it by more than 2^8:
-      // p stays <= 256, exact in fp32 accumulation and harmless in the 16-bit P, and the
-      // rescale of O is skipped on almost every tile.
-      if (__any(mx > m + 8.f)) {
-        const float m_new = fmaxf(m, mx);
-        const float alpha = fast_exp2(m - ((m_new == kNegInf) ? 0.f : m_new));
-        l *= alpha;
-        m = m_new;
-#pragma unroll
-        for (int d = 0; d < DB; d++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) o[d][i] *= alpha;
-      }
-      const float neg_m = (m == kNegInf) ? 0.f : -m;
-      float rs = 0.f;
-      i32x4 P[4];
-      if (need_mask) {
-#pragma unroll
-        for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int c = col0 + 32 * bb + acc_row(i, g);
-            const float p = (c >= lo && c < hi) ? fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m)) : 0.f;
-            s[bb][i] = p;
-            rs += p;
-          }
-      } else {
-#pragma unroll
-        for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m));
-            s[bb][i] = p;
-            rs += p;
-          }
-      }
-#pragma unroll
-      for (int ks = 0; ks < 4; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
-      rs += xor32(rs);
-      l += rs;
-      pv.run(oa, Vs[cur], P, o);
+      lds_cptr Kc = smem + c_st * 2 * BN * HD;
+      tile(std::true_type{}, Kc, Kc + BN * HD, col0, lo, hi);
     }
-
-    ld.wait_all();
+    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    wait_tile(it + 1);
     __syncthreads();
   }
 
@@ -198,7 +230,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const KArgs a) {
 
 template <typename T, int HD>
 hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = 4 * 64 * HD * sizeof(uint16_t);
+  constexpr size_t smem = (size_t)kRowStages * 2 * 64 * HD * sizeof(uint16_t);
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<T, HD>),
@@ -206,11 +238,16 @@ hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  const int64_t nblk = (int64_t)a.nqt * a.B * a.Hq;
+  const int64_t nblk = (int64_t)((a.Tq + kRowBM - 1) / kRowBM) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((fwd_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), smem, stream, a);
+  hipLaunchKernelGGL((fwd_kernel<T, HD>), dim3((unsigned)nblk), dim3(64 * kRowWaves), smem, stream, a);
   return hipGetLastError();
 }
+
+template __global__ void fwd_kernel<BF16, 128>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64>(const KArgs);
 
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_fwd_t<BF16, 128>(a, stream);

@@ -301,6 +301,33 @@ struct AsyncTileLoader {
     row_in_pass = wave * RPW + lane / CH;
     gchunk = (lane % CH) ^ Tile<HD>::swz(row_in_pass);
   }
+  // A source of rows: fixed descriptor over rows [row_base, row_end) of a (batch, head) slice.
+  struct Source {
+    const uint16_t* base;  // row `row_base` of the slice
+    uint32_t nbytes;       // bytes from there to the end of the slice (clamped to 4 GiB)
+    int voff;              // this lane's byte offset inside a tile
+    int stride_bytes;
+    int row_base;
+  };
+  __device__ __forceinline__ Source source(const uint16_t* slice, int64_t row_stride, int row_base, int row_end) const {
+    Source s;
+    s.stride_bytes = (int)row_stride * 2;
+    s.row_base = row_base;
+    const int64_t nbytes = (int64_t)(row_end > row_base ? row_end - row_base : 0) * s.stride_bytes;
+    s.base = slice + (int64_t)row_base * row_stride;
+    s.nbytes = nbytes > 0xffffffffll ? 0xffffffffu : (uint32_t)nbytes;
+    s.voff = row_in_pass * s.stride_bytes + gchunk * 16;
+    return s;
+  }
+  // rows [row0, row0 + ROWS) of the source into `tile`; rows past the source's end arrive as zeros
+  __device__ __forceinline__ void load_from(lds_ptr tile, const Source& s, int row0) const {
+    const int soff = (row0 - s.row_base) * s.stride_bytes;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(s.base, s.nbytes);
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(tile + (i * NW + wave) * 512), 16, s.voff,
+                                               soff + i * NW * RPW * s.stride_bytes, 0, 0);
+  }
   __device__ __forceinline__ void load(lds_ptr tile, const uint16_t* src, int64_t row_stride, int row0,
                                        int row_end) const {
     const int rows_left = row_end - row0;
@@ -315,10 +342,63 @@ struct AsyncTileLoader {
   }
   // s_waitcnt vmcnt(0): every outstanding vector-memory load of this wave has landed
   __device__ __forceinline__ static void wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+  // s_waitcnt vmcnt(K): at most K of this wave's vector-memory loads (the youngest ones) still in flight
+  template <int K>
+  __device__ __forceinline__ static void wait_but() {
+    static_assert(K >= 0 && K < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (K & 15) | ((K >> 4) << 14));
+  }
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+
+// Combine a value with the one held by lane ^ 32 (the other half of the lane pair that shares a
+// row or column) using the gfx950 half-wave swap: {r0, r1} = {x[lane], x[lane ^ 32]} in every lane.
+__device__ __forceinline__ float pair_max(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int xi = __builtin_bit_cast(int, x);
+  auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  return fmaxf(__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1]));
+#else
+  return x;  // host pass of the single-source compile: never executed
+#endif
+}
+__device__ __forceinline__ float pair_sum(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int xi = __builtin_bit_cast(int, x);
+  auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+#else
+  return x;  // host pass of the single-source compile: never executed
+#endif
+}
+
+// acc + (sum of the two 16-bit values packed in w), fp32 accumulation: one instruction per pair.
+template <typename T>
+__device__ __forceinline__ float add_pair(int w, float acc);
+template <>
+__device__ __forceinline__ float add_pair<BF16>(int w, float acc) {
+  bf16x2 ones;
+  ones[0] = (__bf16)1.0f;
+  ones[1] = (__bf16)1.0f;
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, acc, false);
+#else
+  return acc;  // host pass of the single-source compile: never executed
+#endif
+}
+template <>
+__device__ __forceinline__ float add_pair<FP16>(int w, float acc) {
+  f16x2 ones;
+  ones[0] = (_Float16)1.0f;
+  ones[1] = (_Float16)1.0f;
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, acc, false);
+#else
+  return acc;  // host pass of the single-source compile: never executed
+#endif
+}
 
 }  // namespace moda
