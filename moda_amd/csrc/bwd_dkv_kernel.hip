@@ -137,6 +137,84 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   ld.wait_all();
   __syncthreads();
 
+  // Query tiles whose rows ALL see ALL 128 columns of this workgroup need no masking and no
+  // visibility test: for a causal sequence tile those are the tiles at or past the last column's
+  // first visible row (padding rows past Tq carry zero Q, dO, lse, delta and contribute nothing);
+  // non-causal sequence tiles are all of that kind; depth tiles never are.
+  int first_free_qt;  // query tiles (relative to qt0) below this index take the masked body
+  if (dep)
+    first_free_qt = nqt;
+  else if (a.causal)
+    first_free_qt = ((min(ncols, c_first + BN) - 1) * a.Gf + BM - 1) / BM - qt0;
+  else
+    first_free_qt = 0;
+  // the last sequence tile may hold padding columns: their K, V are zero, their results unused
+
+  // role A, one tile: S = Q K^T, P = exp2(S c - lse) -> mailbox, dV^T += dO^T P
+  auto tile_a = [&](auto masked, lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* lse_s, MODA_LDS i32x4* mb,
+                    int q0) {
+    constexpr bool MASKED = decltype(masked)::value;
+    f32x16 s[2];
+    mfma_rows<T, HD, 2, 4>(oa, Qs, Sr, s);
+    TrPipe<T, HD, 4, 2> dvp;
+    dvp.prefetch(oa, dOs);
+#pragma unroll
+    for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int row0 = 32 * bb + 8 * i4 + 4 * g;
+        const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const int i = 4 * i4 + j;
+          float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lv[j]));
+          if (MASKED) {
+            const int qr = q0 + row0 + j;
+            p = (qr >= qlo && qr < qhi) ? p : 0.f;
+          }
+          s[bb][i] = p;
+        }
+      }
+    i32x4 P[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+      mb[ks * 64] = P[ks];
+    }
+    dvp.run(oa, dOs, P, acc);
+  };
+  // role B, one tile: dP = dO V^T, dS = P (dP - delta), dK^T += Q^T dS
+  auto tile_b = [&](lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* del_s, MODA_LDS const i32x4* mb) {
+    f32x16 dp[2];
+    mfma_rows<T, HD, 2, 4>(oa, dOs, Sr, dp);
+    TrPipe<T, HD, 4, 2> dkp;
+    dkp.prefetch(oa, Qs);
+    i32x4 DS[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      const int bb = ks >> 1;
+      const i32x4 pw = mb[ks * 64];
+      // accumulator registers 8*(ks&1) .. +7 of block bb: rows 32bb + 16(ks&1) + {0,8} + 4g + {0..3}
+      const int rbase = 32 * bb + 16 * (ks & 1) + 4 * g;
+      const f32x4 d0 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase);
+      const f32x4 d1 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase + 8);
+      float p[8];
+#pragma unroll
+      for (int w = 0; w < 4; w++) unpack2<T>(pw[w], p[2 * w], p[2 * w + 1]);
+      float ds[8];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        ds[j] = p[j] * (dp[bb][8 * (ks & 1) + j] - d0[j]);
+        ds[4 + j] = p[4 + j] * (dp[bb][8 * (ks & 1) + 4 + j] - d1[j]);
+      }
+      DS[ks][0] = pack2<T>(ds[0], ds[1]);
+      DS[ks][1] = pack2<T>(ds[2], ds[3]);
+      DS[ks][2] = pack2<T>(ds[4], ds[5]);
+      DS[ks][3] = pack2<T>(ds[6], ds[7]);
+    }
+    dkp.run(oa, Qs, DS, acc);
+  };
+
   // consumer cursor of this wave's role: query tile c_qt, ring stage c_st, mailbox parity c_par.
   // Role A handles tile `it`, role B tile `it - 1`; one extra trip drains B.
   int c_qt = 0, c_st = 0, c_par = 0;
@@ -145,92 +223,22 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     const bool active = role_b ? (it >= 1) : (it < niter);
     if (active) {
       const int q0 = (qt0 + c_qt) * BM;
-      const bool touches = (qhi > q0) && (qlo < q0 + BM) && (qhi > qlo);
-      if (__any(touches)) {
-        lds_cptr Qs = ring + c_st * 2 * BM * HD;
-        lds_cptr dOs = Qs + BM * HD;
-        MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * 4 * 64 + lane;
-        if (!role_b) {
-          const bool full = (qlo <= q0) && (qhi >= q0 + BM);
-          MODA_LDS const float* lse_s = stat + c_st * 2 * BM;
-          f32x16 s[2];
-#pragma unroll
-          for (int bb = 0; bb < 2; bb++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) s[bb][i] = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < KK; kk++) s[bb] = mfma32<T>(oa.row_operand(Qs, 32 * bb, kk), Sr[kk], s[bb]);
-          }
-          auto probs = [&](auto masked) {
-#pragma unroll
-            for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-              for (int i4 = 0; i4 < 4; i4++) {
-                const int row0 = 32 * bb + 8 * i4 + 4 * g;
-                const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                  const int i = 4 * i4 + j;
-                  float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lv[j]));
-                  if (decltype(masked)::value) {
-                    const int qr = q0 + row0 + j;
-                    p = (qr >= qlo && qr < qhi) ? p : 0.f;
-                  }
-                  s[bb][i] = p;
-                }
-              }
-          };
-          if (__all(full))
-            probs(std::false_type{});
+      lds_cptr Qs = ring + c_st * 2 * BM * HD;
+      lds_cptr dOs = Qs + BM * HD;
+      MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * 4 * 64 + lane;
+      MODA_LDS const float* st_s = stat + c_st * 2 * BM;
+      if (c_qt >= first_free_qt) {
+        if (!role_b)
+          tile_a(std::false_type{}, Qs, dOs, st_s, mb, q0);
+        else
+          tile_b(Qs, dOs, st_s + BM, mb);
+      } else {
+        const bool touches = (qhi > q0) && (qlo < q0 + BM) && (qhi > qlo);
+        if (__any(touches)) {
+          if (!role_b)
+            tile_a(std::true_type{}, Qs, dOs, st_s, mb, q0);
           else
-            probs(std::true_type{});
-          i32x4 P[4];
-#pragma unroll
-          for (int ks = 0; ks < 4; ks++) {
-            P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
-            mb[ks * 64] = P[ks];
-          }
-#pragma unroll
-          for (int d = 0; d < DB; d++)
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) acc[d] = mfma32<T>(oa.tr_operand(dOs, 16 * ks, d), P[ks], acc[d]);
-        } else {
-          MODA_LDS const float* del_s = stat + c_st * 2 * BM + BM;
-          f32x16 dp[2];
-#pragma unroll
-          for (int bb = 0; bb < 2; bb++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) dp[bb][i] = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < KK; kk++) dp[bb] = mfma32<T>(oa.row_operand(dOs, 32 * bb, kk), Sr[kk], dp[bb]);
-          }
-          i32x4 DS[4];
-#pragma unroll
-          for (int ks = 0; ks < 4; ks++) {
-            const int bb = ks >> 1;
-            const i32x4 pw = mb[ks * 64];
-            // accumulator registers 8*(ks&1) .. +7 of block bb: rows 32bb + 16(ks&1) + {0,8} + 4g + {0..3}
-            const int rbase = 32 * bb + 16 * (ks & 1) + 4 * g;
-            const f32x4 d0 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase);
-            const f32x4 d1 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase + 8);
-            float p[8];
-#pragma unroll
-            for (int w = 0; w < 4; w++) unpack2<T>(pw[w], p[2 * w], p[2 * w + 1]);
-            float ds[8];
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-              ds[j] = p[j] * (dp[bb][8 * (ks & 1) + j] - d0[j]);
-              ds[4 + j] = p[4 + j] * (dp[bb][8 * (ks & 1) + 4 + j] - d1[j]);
-            }
-            DS[ks][0] = pack2<T>(ds[0], ds[1]);
-            DS[ks][1] = pack2<T>(ds[2], ds[3]);
-            DS[ks][2] = pack2<T>(ds[4], ds[5]);
-            DS[ks][3] = pack2<T>(ds[6], ds[7]);
-          }
-#pragma unroll
-          for (int d = 0; d < DB; d++)
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) acc[d] = mfma32<T>(oa.tr_operand(Qs, 16 * ks, d), DS[ks], acc[d]);
+            tile_b(Qs, dOs, st_s + BM, mb);
         }
       }
       if (++c_qt == nqt) c_qt = 0;
@@ -282,6 +290,11 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((dkv_kernel<T, HD>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
   return hipGetLastError();
 }
+
+template __global__ void dkv_kernel<BF16, 128>(const KArgs);
+template __global__ void dkv_kernel<BF16, 64>(const KArgs);
+template __global__ void dkv_kernel<FP16, 128>(const KArgs);
+template __global__ void dkv_kernel<FP16, 64>(const KArgs);
 
 hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_dkv_t<BF16, 128>(a, stream);

@@ -7,6 +7,8 @@
 // the rows' depth slots).  P^T is recomputed from the saved base-2 LSE,
 // dS^T = P^T * (dP^T - delta) is packed straight into the B operand of
 // dQ^T += K^T * dS^T, K^T coming from the LDS transpose read of the K tile.
+#include <type_traits>
+
 #include "kargs.h"
 #include "tile.h"
 #include "tuning.h"
@@ -83,8 +85,13 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const
   const int r_first = qt * BM;
   const int r_last = min(a.Tq, r_first + BM) - 1;
   const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
-  int n_seq = 0;
-  if (a.has_seq) n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
+  int n_seq = 0, n_full = 0;
+  if (a.has_seq) {
+    n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
+    // leading sequence tiles every row of the workgroup sees completely (padding rows of the last
+    // workgroup carry zero queries and zero dO there and are never stored)
+    n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
+  }
   int dep0 = 0, n_dep = 0;
   if (a.L > 0) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
@@ -93,27 +100,27 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const
   }
   const int ntiles = n_seq + n_dep;
 
-  const uint16_t* kb = a.has_seq ? a.k + b * a.sk.b + hkv * a.sk.h : nullptr;
-  const uint16_t* vb = a.has_seq ? a.v + b * a.sv.b + hkv * a.sv.h : nullptr;
-  const uint16_t* kdb = a.L > 0 ? a.kd + b * a.skd.b + hkv * a.skd.h : nullptr;
-  const uint16_t* vdb = a.L > 0 ? a.vd + b * a.svd.b + hkv * a.svd.h : nullptr;
-  const int TL = a.T * a.L;
-
   typedef AsyncTileLoader<HD, BN, NT> Loader;
   constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
   Loader ld;
   ld.init(tid);
+  // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
+  // producer reaches the first depth tile
+  typename Loader::Source srcK, srcV;
+  if (a.has_seq && n_seq > 0) {
+    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
+    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
+  }
   int ld_st = 0;  // ring stage the next issued tile goes to
   auto issue = [&](int it) {
     lds_ptr Kt = smem + ld_st * 2 * BN * HD;
-    if (it < n_seq) {
-      ld.load(Kt, kb, a.sk.t, it * BN, a.T);
-      ld.load(Kt + BN * HD, vb, a.sv.t, it * BN, a.T);
-    } else {
-      const int c0 = dep0 + (it - n_seq) * BN;
-      ld.load(Kt, kdb, a.skd.t, c0, TL);
-      ld.load(Kt + BN * HD, vdb, a.svd.t, c0, TL);
+    if (it == n_seq) {
+      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
+      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
+    const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
+    ld.load_from(Kt, srcK, row0);
+    ld.load_from(Kt + BN * HD, srcV, row0);
     ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
   };
   // wait until tile `next` has landed; tiles next+1 .. next+DIST-1 may still be in flight
@@ -140,54 +147,51 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const
   __syncthreads();
   int c_st = 0;  // ring stage of the tile being consumed
 
-  for (int it = 0; it < ntiles; it++) {
+  // one column tile: S^T = K Q^T and dP^T = V dO^T in one MFMA pipeline, dS^T, dQ^T += K^T dS^T
+  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, int lo, int hi) {
+    constexpr bool MASKED = decltype(masked)::value;
+    f32x16 s[2], dp[2];
+    mfma_rows2<T, HD, 2, 4>(oa, Kc, Qr, s, Vc, dOr, dp);
+    TrPipe<T, HD, 4, 2> kt;
+    kt.prefetch(oa, Kc);
+#pragma unroll
+    for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lse));
+        if (MASKED) {
+          const int c = col0 + 32 * bb + acc_row(i, g);
+          p = (c >= lo && c < hi) ? p : 0.f;
+        }
+        s[bb][i] = p * (dp[bb][i] - delta);
+      }
+    i32x4 DS[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) DS[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+    kt.run(oa, Kc, DS, dq);
+  };
+
+  // phase 1: tiles fully visible to every row -- no masks, no visibility tests
+  for (int it = 0; it < n_full; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     lds_cptr Kc = smem + c_st * 2 * BN * HD;
-    lds_cptr Vc = Kc + BN * HD;
-
+    tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, 0, 0);
+    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    wait_tile(it + 1);
+    __syncthreads();
+  }
+  // phase 2: boundary sequence tiles and depth tiles
+  for (int it = n_full; it < ntiles; it++) {
+    if (it + DIST < ntiles) issue(it + DIST);
     const bool dep = it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
     const int lo = dep ? dlo : 0;
     const int hi = dep ? dhi : shi;
     const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
     if (__any(touches)) {
-      const bool full = (lo <= col0) && (hi >= col0 + BN);
-      const bool need_mask = !__all(full);
-      f32x16 s[2], dp[2];
-#pragma unroll
-      for (int bb = 0; bb < 2; bb++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          s[bb][i] = 0.f;
-          dp[bb][i] = 0.f;
-        }
-#pragma unroll
-        for (int kk = 0; kk < KK; kk++) {
-          s[bb] = mfma32<T>(oa.row_operand(Kc, 32 * bb, kk), Qr[kk], s[bb]);
-          dp[bb] = mfma32<T>(oa.row_operand(Vc, 32 * bb, kk), dOr[kk], dp[bb]);
-        }
-      }
-#pragma unroll
-      for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          float p = fast_exp2(s[bb][i] * sc - lse);
-          if (need_mask) {
-            const int c = col0 + 32 * bb + acc_row(i, g);
-            p = (c >= lo && c < hi) ? p : 0.f;
-          }
-          s[bb][i] = p * (dp[bb][i] - delta);
-        }
-      i32x4 DS[4];
-#pragma unroll
-      for (int ks = 0; ks < 4; ks++) DS[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
-#pragma unroll
-      for (int d = 0; d < DB; d++)
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++)
-          dq[d] = mfma32<T>(oa.tr_operand(Kc, 16 * ks, d), DS[ks], dq[d]);
+      lds_cptr Kc = smem + c_st * 2 * BN * HD;
+      tile(std::true_type{}, Kc, Kc + BN * HD, col0, lo, hi);
     }
-
     c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
     wait_tile(it + 1);
     __syncthreads();
@@ -230,6 +234,11 @@ hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((dq_kernel<T, HD>), dim3((unsigned)nblk), dim3(64 * kRowWaves), smem, stream, a);
   return hipGetLastError();
 }
+
+template __global__ void dq_kernel<BF16, 128>(const KArgs);
+template __global__ void dq_kernel<BF16, 64>(const KArgs);
+template __global__ void dq_kernel<FP16, 128>(const KArgs);
+template __global__ void dq_kernel<FP16, 64>(const KArgs);
 
 hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_delta_t<BF16, 128>(a, stream);
