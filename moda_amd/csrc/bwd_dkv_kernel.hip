@@ -5,7 +5,9 @@
 // A workgroup (eight waves) owns 128 key columns of one (batch, kv head) --
 // sequence keys or flattened depth slots -- as four 32-column blocks, one column
 // per lane pair.  It streams 64-row query tiles (Q, dO, LSE, delta) through a
-// three-stage LDS ring over exactly the query rows that can see its columns:
+// three-stage LDS ring, from the last tile down to its diagonal (workgroups that
+// run together then read the same tiles at the same time and share them in L2),
+// over exactly the query rows that can see its columns:
 // all later tokens for a causal sequence key, the owner token's G rows (or the
 // rest of its chunk) for a depth slot.  Two waves share each column block and
 // split the work by ROLE so that each stays under 256 registers and the two
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   // producer cursor: next tile to fetch = (query head ld_gh, query tile ld_qt) into ring stage ld_st
   int ld_qt = 0, ld_gh = 0, ld_st = 0;
   auto issue = [&]() {
-    const int q0 = (qt0 + ld_qt) * BM;
+    const int q0 = (qt0 + nqt - 1 - ld_qt) * BM;  // tiles are walked from the last one down
     const int hq = hkv * a.hdiv + ld_gh;
     lds_ptr stage = ring + ld_st * 2 * BM * HD;
     ld.load(stage, a.q + b * a.sq.b + hq * a.sq.h, a.sq.t, q0, a.Tq);
@@ -222,12 +224,13 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     if (it + 1 < niter) issue();
     const bool active = role_b ? (it >= 1) : (it < niter);
     if (active) {
-      const int q0 = (qt0 + c_qt) * BM;
+      const int rel_qt = nqt - 1 - c_qt;
+      const int q0 = (qt0 + rel_qt) * BM;
       lds_cptr Qs = ring + c_st * 2 * BM * HD;
       lds_cptr dOs = Qs + BM * HD;
       MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * 4 * 64 + lane;
       MODA_LDS const float* st_s = stat + c_st * 2 * BM;
-      if (c_qt >= first_free_qt) {
+      if (rel_qt >= first_free_qt) {
         if (!role_b)
           tile_a(std::false_type{}, Qs, dOs, st_s, mb, q0);
         else
