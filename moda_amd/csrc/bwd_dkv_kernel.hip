@@ -77,6 +77,13 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     }
   }
 
+  // The register operands above must have arrived before the tile loads start: those are issued
+  // behind the compiler's back, and a load it still believes pending would cost a vmcnt(0) in every
+  // trip of the main loop.
+  asm volatile("" ::: "memory");  // keep the loads above this point
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("" ::: "memory");
+
   // visible query-row interval of a column
   auto q_interval = [&](int col, int& lo, int& hi) {
     if (!dep) {
@@ -110,14 +117,12 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     // per-row statistics straight into LDS as well: wave 0 fetches lse, wave 1 delta (one dword per lane)
     const int rows = min(a.Tq - q0, BM);
     if (wave == 0) {
-      const __amdgpu_buffer_rsrc_t rs =
-          make_rsrc(a.lse + ((int64_t)b * a.Tq + q0) * a.Hq + hq, rows > 0 ? ((rows - 1) * a.Hq + 1) * 4u : 0u);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(stat + ld_st * 2 * BM), 4, lane * a.Hq * 4, 0, 0,
-                                               0);
+      const i32x4 rs =
+          rsrc_words(a.lse + ((int64_t)b * a.Tq + q0) * a.Hq + hq, rows > 0 ? ((rows - 1) * a.Hq + 1) * 4u : 0u);
+      lds_dma<4>(rs, (uint32_t)(uintptr_t)(stat + ld_st * 2 * BM), lane * a.Hq * 4, 0);
     } else if (wave == 1) {
-      const __amdgpu_buffer_rsrc_t rs =
-          make_rsrc(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + q0, rows > 0 ? rows * 4u : 0u);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(stat + ld_st * 2 * BM + BM), 4, lane * 4, 0, 0, 0);
+      const i32x4 rs = rsrc_words(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + q0, rows > 0 ? rows * 4u : 0u);
+      lds_dma<4>(rs, (uint32_t)(uintptr_t)(stat + ld_st * 2 * BM + BM), lane * 4, 0);
     }
     if (++ld_qt == nqt) {
       ld_qt = 0;
@@ -185,10 +190,19 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     }
     dvp.run(oa, dOs, P, acc);
   };
-  // role B, one tile: dP = dO V^T, dS = P (dP - delta), dK^T += Q^T dS
+  // role B, one tile: dP - delta = dO V^T with the accumulators preset to -delta (the workspace holds
+  // minus delta), dS = P (dP - delta), dK^T += Q^T dS
   auto tile_b = [&](lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* del_s, MODA_LDS const i32x4* mb) {
     f32x16 dp[2];
-    mfma_rows<T, HD, 2, 4>(oa, dOs, Sr, dp);
+#pragma unroll
+    for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const f32x4 dv = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + 32 * bb + 8 * i4 + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; j++) dp[bb][4 * i4 + j] = dv[j];
+      }
+    mfma_rows_acc<T, HD, 2, 4>(oa, dOs, Sr, dp);
     TrPipe<T, HD, 4, 2> dkp;
     dkp.prefetch(oa, Qs);
     i32x4 DS[4];
@@ -196,23 +210,12 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     for (int ks = 0; ks < 4; ks++) {
       const int bb = ks >> 1;
       const i32x4 pw = mb[ks * 64];
-      // accumulator registers 8*(ks&1) .. +7 of block bb: rows 32bb + 16(ks&1) + {0,8} + 4g + {0..3}
-      const int rbase = 32 * bb + 16 * (ks & 1) + 4 * g;
-      const f32x4 d0 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase);
-      const f32x4 d1 = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + rbase + 8);
       float p[8];
 #pragma unroll
       for (int w = 0; w < 4; w++) unpack2<T>(pw[w], p[2 * w], p[2 * w + 1]);
-      float ds[8];
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        ds[j] = p[j] * (dp[bb][8 * (ks & 1) + j] - d0[j]);
-        ds[4 + j] = p[4 + j] * (dp[bb][8 * (ks & 1) + 4 + j] - d1[j]);
-      }
-      DS[ks][0] = pack2<T>(ds[0], ds[1]);
-      DS[ks][1] = pack2<T>(ds[2], ds[3]);
-      DS[ks][2] = pack2<T>(ds[4], ds[5]);
-      DS[ks][3] = pack2<T>(ds[6], ds[7]);
+      for (int w = 0; w < 4; w++)
+        DS[ks][w] = pack2<T>(p[2 * w] * dp[bb][8 * (ks & 1) + 2 * w], p[2 * w + 1] * dp[bb][8 * (ks & 1) + 2 * w + 1]);
     }
     dkp.run(oa, Qs, DS, acc);
   };

@@ -1,4 +1,4 @@
-// Backward, query side: delta = rowsum(o * do) (moda_v14.py:525-539) and the
+// Backward, query side: the preprocess kernel (-delta = -rowsum(o * do), moda_v14.py:525-539) and the
 // dQ kernel (moda_v14.py:542-871, moda_v16.py:936-1220, fda_v12.py:432-638,
 // fla/ops/attn/parallel.py:165-296).
 //
@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a) {
   }
 #pragma unroll
   for (int s = TPR / 2; s > 0; s >>= 1) acc += __shfl_xor(acc, s, 64);
-  if (r < a.Tq && (tid % TPR) == 0) a.delta[((int64_t)b * a.Hq + hq) * a.Tq + r] = acc;
+  if (r < a.Tq && (tid % TPR) == 0) a.delta[((int64_t)b * a.Hq + hq) * a.Tq + r] = -acc;
 }
 
 template <typename T, int HD>
@@ -72,6 +72,13 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const
       delta = a.delta[((int64_t)b * a.Hq + hq) * a.Tq + r];
     }
   }
+
+  // The register operands above must have arrived before the tile loads start: those are issued
+  // behind the compiler's back, and a load it still believes pending would cost a vmcnt(0) in every
+  // trip of the main loop.
+  asm volatile("" ::: "memory");  // keep the loads above this point
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("" ::: "memory");
 
   int shi = 0, dlo = 0, dhi = 0;
   if (valid) {
@@ -163,7 +170,7 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const
           const int c = col0 + 32 * bb + acc_row(i, g);
           p = (c >= lo && c < hi) ? p : 0.f;
         }
-        s[bb][i] = p * (dp[bb][i] - delta);
+        s[bb][i] = p * (dp[bb][i] + delta);  // delta holds minus rowsum(o * do)
       }
     i32x4 DS[4];
 #pragma unroll

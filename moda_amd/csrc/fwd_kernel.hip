@@ -50,6 +50,13 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void fwd_kernel(cons
     }
   }
 
+  // The register operands above must have arrived before the tile loads start: those are issued
+  // behind the compiler's back, and a load it still believes pending would cost a vmcnt(0) in every
+  // trip of the main loop.
+  asm volatile("" ::: "memory");  // keep the loads above this point
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("" ::: "memory");
+
   // per-row visible column intervals [lo, hi) for the two phases
   int shi = 0, dlo = 0, dhi = 0;
   if (valid) {

@@ -12,7 +12,7 @@ struct KArgs {
   const uint16_t *q, *k, *v, *kd, *vd, *o, *d_o;
   uint16_t *out_o, *dq, *dk, *dv, *dkd, *dvd;
   float* lse;          // [B, Tq, Hq]   (written by forward, read by backward)
-  float* delta;        // [B, Hq, Tq]   workspace
+  float* delta;        // [B, Hq, Tq]   workspace: MINUS rowsum(o * do)
   Str3 sq, sk, sv, skd, svd, so, sdo, sdq, sdk, sdv, sdkd, sdvd;
   int B, T, Hkv;
   int Tq;    // query rows per (batch, query head)

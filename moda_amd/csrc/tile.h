@@ -186,6 +186,23 @@ __device__ __forceinline__ void mfma_rows(const OperandAddr<HD>& oa, lds_cptr ti
   }
 }
 
+// acc[bb] += sum_kk rows(tile, 32*bb + n, kk) x breg[kk]   (accumulators preset by the caller)
+template <typename T, int HD, int NB, int DEPTH>
+__device__ __forceinline__ void mfma_rows_acc(const OperandAddr<HD>& oa, lds_cptr tile, const i32x4 (&breg)[HD / 16],
+                                              f32x16 (&acc)[NB]) {
+  constexpr int KK = HD / 16, N = NB * KK;
+  i32x4 ops[N];
+#pragma unroll
+  for (int j = 0; j < DEPTH && j < N; j++) ops[j] = oa.row_operand(tile, 32 * (j % NB), j / NB);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < N; j++) {
+    if (j + DEPTH < N) ops[j + DEPTH] = oa.row_operand(tile, 32 * ((j + DEPTH) % NB), (j + DEPTH) / NB);
+    acc[j % NB] = mfma32<T>(ops[j], breg[j / NB], acc[j % NB]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 // Two tiles against two register operands in one pipeline:
 // acc0[bb] = rows(tile0) x breg0, acc1[bb] = rows(tile1) x breg1.
 template <typename T, int HD, int NB, int DEPTH>
@@ -278,6 +295,42 @@ struct TileLoader {
   }
 };
 
+// One wave-wide direct global -> LDS load: lane l's BYTES bytes (16 or 4) land at lds_byte_addr +
+// l * BYTES; the global side is a raw buffer (descriptor rsrc, per-lane byte offset voff, scalar
+// byte offset soff) whose range check zero-fills lanes past the end.  Issued as inline assembly on
+// purpose: the compiler's wait-count pass does not see these loads, so it does not stall every
+// later LDS read (in particular the transpose reads) on vmcnt(0) while the NEXT tiles are still in
+// flight.  Completion is the caller's business: s_waitcnt vmcnt via wait_all()/wait_but<>() and a
+// workgroup barrier before any wave reads the tile.  The compiler's own vmcnt waits stay correct
+// because vector-memory loads return in order and an unseen younger load only makes them stricter.
+template <int BYTES>
+__device__ __forceinline__ void lds_dma(i32x4 rsrc, uint32_t lds_byte_addr, int voff, int soff) {
+  static_assert(BYTES == 16 || BYTES == 4, "dwordx4 or dword");
+  if (BYTES == 16)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory", "m0");
+}
+
+// The four descriptor words of a raw buffer over `nbytes` bytes at `base` (wave-uniform).
+__device__ __forceinline__ i32x4 rsrc_words(const void* base, uint32_t nbytes) {
+  const uint64_t p = (uint64_t)base;
+  i32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+  r[1] = __builtin_amdgcn_readfirstlane((int)((uint32_t)(p >> 32) & 0xffffu));
+  r[2] = __builtin_amdgcn_readfirstlane((int)nbytes);
+  r[3] = 0x00020000;
+  return r;
+}
+
+__device__ __forceinline__ uint32_t lds_addr(lds_cptr p) { return (uint32_t)(uintptr_t)p; }
+
 // Global -> LDS staging without registers: gfx950 `buffer_load_dwordx4 ... lds`.
 // One wave-wide load fills 64 consecutive 16-byte LDS slots (lane l -> slot l);
 // the XOR swizzle is therefore applied on the GLOBAL side: the lane that owns
@@ -322,23 +375,21 @@ struct AsyncTileLoader {
   // rows [row0, row0 + ROWS) of the source into `tile`; rows past the source's end arrive as zeros
   __device__ __forceinline__ void load_from(lds_ptr tile, const Source& s, int row0) const {
     const int soff = (row0 - s.row_base) * s.stride_bytes;
-    const __amdgpu_buffer_rsrc_t rs = make_rsrc(s.base, s.nbytes);
+    const i32x4 rs = rsrc_words(s.base, s.nbytes);
 #pragma unroll
     for (int i = 0; i < N; i++)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(tile + (i * NW + wave) * 512), 16, s.voff,
-                                               soff + i * NW * RPW * s.stride_bytes, 0, 0);
+      lds_dma<16>(rs, lds_addr(tile + (i * NW + wave) * 512), s.voff, soff + i * NW * RPW * s.stride_bytes);
   }
   __device__ __forceinline__ void load(lds_ptr tile, const uint16_t* src, int64_t row_stride, int row0,
                                        int row_end) const {
     const int rows_left = row_end - row0;
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const uint32_t nbytes = rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
-    const __amdgpu_buffer_rsrc_t rs = make_rsrc(src + (int64_t)row0 * row_stride, nbytes);
+    const i32x4 rs = rsrc_words(src + (int64_t)row0 * row_stride, nbytes);
     const int voff = row_in_pass * (int)stride_bytes + gchunk * 16;
 #pragma unroll
     for (int i = 0; i < N; i++)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (MODA_LDS void*)(tile + (i * NW + wave) * 512), 16, voff,
-                                               i * NW * RPW * (int)stride_bytes, 0, 0);
+      lds_dma<16>(rs, lds_addr(tile + (i * NW + wave) * 512), voff, i * NW * RPW * (int)stride_bytes);
   }
   // s_waitcnt vmcnt(0): every outstanding vector-memory load of this wave has landed
   __device__ __forceinline__ static void wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
