@@ -89,8 +89,9 @@ int moda_hip_fwd(const moda_hip_desc* desc, const void* q, const void* k, const 
                  const void* kd, const void* vd, void* o, float* lse, void* stream);
 
 /*
- * Bytes of device workspace moda_hip_bwd needs (holds delta = rowsum(o * do),
- * the quantity of moda_v14.py:525-539).  Returns 0 for an invalid descriptor.
+ * Bytes of device workspace moda_hip_bwd needs (one fp32 per query row and
+ * head: the row sum of o * do of moda_v14.py:525-539, kept in a form private to
+ * the library).  Returns 0 for an invalid descriptor.
  */
 size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* desc);
 
@@ -117,7 +118,7 @@ int moda_hip_bwd(const moda_hip_desc* desc, const void* q, const void* k, const 
  * 1698-1801).
  */
 enum moda_hip_bwd_stage {
-  MODA_HIP_STAGE_DELTA = 1, /* delta = rowsum(o * do)                 */
+  MODA_HIP_STAGE_DELTA = 1, /* row sums of o * do into the workspace  */
   MODA_HIP_STAGE_DQ = 2,    /* dq                                     */
   MODA_HIP_STAGE_DKV = 4,   /* dk, dv and, with a depth stream, dkd, dvd */
   MODA_HIP_STAGE_ALL = 7

@@ -89,8 +89,10 @@ def test_reference_matrix(gpu_device, idx):
         if ref[n] is None:
             continue
         assert oracle.passes_reference_rule(got[n].float().cpu(), ref[n]), (idx, n)
-        _, l2 = oracle.error_metrics(got[n].float().cpu(), ref[n])
-        assert l2 <= 1e-2, (idx, n, l2)
+        # tighter than the reference's rule; the absolute alternative covers tensors whose true value is
+        # (numerically) zero, e.g. dk of a one-token sequence, where a relative error means nothing
+        max_abs, l2 = oracle.error_metrics(got[n].float().cpu(), ref[n])
+        assert l2 <= 1e-2 or max_abs <= 1e-3, (idx, n, l2, max_abs)
     check("lse", got["lse"], ref["lse"], dtype, f"matrix {idx}")
 
 
