@@ -5,9 +5,10 @@
 // A workgroup (eight waves) owns 128 key columns of one (batch, kv head) --
 // sequence keys or flattened depth slots -- as four 32-column blocks, one column
 // per lane pair.  It streams 64-row query tiles (Q, dO, LSE, delta) through a
-// three-stage LDS ring, from the last tile down to its diagonal (workgroups that
-// run together then read the same tiles at the same time and share them in L2),
-// over exactly the query rows that can see its columns:
+// three-stage LDS ring (one tile in flight while each role consumes one), from
+// the last tile down to its
+// diagonal (workgroups that run together then read the same tiles at the same
+// time and share them in L2), over exactly the query rows that can see its columns:
 // all later tokens for a causal sequence key, the owner token's G rows (or the
 // rest of its chunk) for a depth slot.  Two waves share each column block and
 // split the work by ROLE so that each stays under 256 registers and the two
@@ -104,31 +105,62 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   const int nqt = (wg_hi + BM - 1) / BM - qt0;
   const int niter = nqt * a.hdiv;
 
-  AsyncTileLoader<HD, BM, 512> ld;
+  using Loader = AsyncTileLoader<HD, BM, 512>;
+  static_assert(Loader::N == HD / 64, "one or two wave-wide loads per tile and wave");
+  Loader ld;
   ld.init(tid);
-  // producer cursor: next tile to fetch = (query head ld_gh, query tile ld_qt) into ring stage ld_st
+  // Producer.  The global -> LDS loads of one tile are NOT issued back to back: forty wave-wide
+  // loads arriving at once queue up in the CU's address unit and every wave would sit on its issue
+  // for hundreds of cycles.  prep() fixes the descriptors of the next tile (wave-uniform, scalar
+  // registers only); part(k), k < kParts, issues one load; the tile bodies slip the parts between
+  // the MFMAs of their first phase, early enough for the tile to land within the trip.  Cursor: next tile = (query head ld_gh, query tile ld_qt) into ring stage ld_st.
+  constexpr int kParts = 2 * Loader::N + 1;
   int ld_qt = 0, ld_gh = 0, ld_st = 0;
-  auto issue = [&]() {
+  i32x4 rs_q, rs_do, rs_stat;
+  uint32_t lds_q, lds_stat;
+  int voff_q, voff_do, voff_stat;
+  auto prep = [&]() {
     const int q0 = (qt0 + nqt - 1 - ld_qt) * BM;  // tiles are walked from the last one down
     const int hq = hkv * a.hdiv + ld_gh;
-    lds_ptr stage = ring + ld_st * 2 * BM * HD;
-    ld.load(stage, a.q + b * a.sq.b + hq * a.sq.h, a.sq.t, q0, a.Tq);
-    ld.load(stage + BM * HD, a.d_o + b * a.sdo.b + hq * a.sdo.h, a.sdo.t, q0, a.Tq);
+    const int rows = max(min(a.Tq - q0, BM), 0);
+    rs_q = rsrc_words(a.q + b * a.sq.b + hq * a.sq.h + (int64_t)q0 * a.sq.t, (uint32_t)rows * (uint32_t)a.sq.t * 2u);
+    rs_do = rsrc_words(a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)q0 * a.sdo.t, (uint32_t)rows * (uint32_t)a.sdo.t * 2u);
+    voff_q = ld.row_in_pass * (int)a.sq.t * 2 + ld.gchunk * 16;
+    voff_do = ld.row_in_pass * (int)a.sdo.t * 2 + ld.gchunk * 16;
+    lds_q = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr(ring + ld_st * 2 * BM * HD + wave * 512));
     // per-row statistics straight into LDS as well: wave 0 fetches lse, wave 1 delta (one dword per lane)
-    const int rows = min(a.Tq - q0, BM);
     if (wave == 0) {
-      const i32x4 rs =
-          rsrc_words(a.lse + ((int64_t)b * a.Tq + q0) * a.Hq + hq, rows > 0 ? ((rows - 1) * a.Hq + 1) * 4u : 0u);
-      lds_dma<4>(rs, (uint32_t)(uintptr_t)(stat + ld_st * 2 * BM), lane * a.Hq * 4, 0);
-    } else if (wave == 1) {
-      const i32x4 rs = rsrc_words(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + q0, rows > 0 ? rows * 4u : 0u);
-      lds_dma<4>(rs, (uint32_t)(uintptr_t)(stat + ld_st * 2 * BM + BM), lane * 4, 0);
+      rs_stat = rsrc_words(a.lse + ((int64_t)b * a.Tq + q0) * a.Hq + hq, rows > 0 ? ((rows - 1) * a.Hq + 1) * 4u : 0u);
+      voff_stat = lane * a.Hq * 4;
+    } else {
+      rs_stat = rsrc_words(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + q0, (uint32_t)rows * 4u);
+      voff_stat = lane * 4;
     }
+    lds_stat = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(stat + ld_st * 2 * BM + (wave == 0 ? 0 : BM)));
     if (++ld_qt == nqt) {
       ld_qt = 0;
       ld_gh++;
     }
     ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
+  };
+  bool feeding = false;  // this trip has a tile to fetch
+  auto part = [&](int k) {
+    if (!feeding) return;
+    __builtin_amdgcn_sched_barrier(0);
+    if (k < Loader::N)
+      lds_dma<16>(rs_q, lds_q + k * 8 * 1024, voff_q, k * 8 * Loader::RPW * (int)a.sq.t * 2);
+    else if (k < 2 * Loader::N)
+      lds_dma<16>(rs_do, lds_q + BM * HD * 2 + (k - Loader::N) * 8 * 1024, voff_do,
+                  (k - Loader::N) * 8 * Loader::RPW * (int)a.sdo.t * 2);
+    else if (wave < 2)
+      lds_dma<4>(rs_stat, lds_stat, voff_stat, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // hook for the first MFMA phase of a tile body: one part after every third MFMA (every second one when
+  // the phase is short)
+  auto feed = [&](int j) {
+    constexpr int every = HD == 128 ? 3 : 2;
+    if (j % every == 1 && j / every < kParts) part(j / every);
   };
 
   f32x16 acc[DB];  // dV^T (role A) or dK^T (role B)
@@ -140,8 +172,11 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   OperandAddr<HD> oa;
   oa.init(lane);
 
-  if (niter > 0) issue();
-  ld.wait_all();
+  feeding = niter > 0;
+  if (feeding) prep();
+#pragma unroll
+  for (int k = 0; k < kParts; k++) part(k);
+  Loader::wait_all();
   __syncthreads();
 
   // Query tiles whose rows ALL see ALL 128 columns of this workgroup need no masking and no
@@ -158,30 +193,28 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   // the last sequence tile may hold padding columns: their K, V are zero, their results unused
 
   // role A, one tile: S = Q K^T, P = exp2(S c - lse) -> mailbox, dV^T += dO^T P
-  auto tile_a = [&](auto masked, lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* lse_s, MODA_LDS i32x4* mb,
-                    int q0) {
-    constexpr bool MASKED = decltype(masked)::value;
+  auto tile_a = [&](bool masked, lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* lse_s, MODA_LDS i32x4* mb, int q0) {
     f32x16 s[2];
-    mfma_rows<T, HD, 2, 4>(oa, Qs, Sr, s);
+    mfma_rows<T, HD, 2, 4>(oa, Qs, Sr, s, feed);
     TrPipe<T, HD, 4, 2> dvp;
     dvp.prefetch(oa, dOs);
 #pragma unroll
     for (int bb = 0; bb < 2; bb++)
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
-        const int row0 = 32 * bb + 8 * i4 + 4 * g;
-        const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + row0);
+        const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + 32 * bb + 8 * i4 + 4 * g);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const int i = 4 * i4 + j;
-          float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lv[j]));
-          if (MASKED) {
-            const int qr = q0 + row0 + j;
-            p = (qr >= qlo && qr < qhi) ? p : 0.f;
-          }
-          s[bb][i] = p;
-        }
+        for (int j = 0; j < 4; j++) s[bb][4 * i4 + j] = fast_exp2(__builtin_fmaf(s[bb][4 * i4 + j], sc, -lv[j]));
       }
+    if (masked) {  // wave-uniform; touches only s, so the accumulators stay where they are
+#pragma unroll
+      for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          const int qr = q0 + 32 * bb + 8 * (i >> 2) + 4 * g + (i & 3);
+          s[bb][i] = (qr >= qlo && qr < qhi) ? s[bb][i] : 0.f;
+        }
+    }
     i32x4 P[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
@@ -202,7 +235,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; j++) dp[bb][4 * i4 + j] = dv[j];
       }
-    mfma_rows_acc<T, HD, 2, 4>(oa, dOs, Sr, dp);
+    mfma_rows_acc<T, HD, 2, 4>(oa, dOs, Sr, dp, feed);
     TrPipe<T, HD, 4, 2> dkp;
     dkp.prefetch(oa, Qs);
     i32x4 DS[4];
@@ -220,40 +253,73 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     dkp.run(oa, Qs, DS, acc);
   };
 
-  // consumer cursor of this wave's role: query tile c_qt, ring stage c_st, mailbox parity c_par.
-  // Role A handles tile `it`, role B tile `it - 1`; one extra trip drains B.
-  int c_qt = 0, c_st = 0, c_par = 0;
-  for (int it = 0; it <= niter; it++) {
-    if (it + 1 < niter) issue();
-    const bool active = role_b ? (it >= 1) : (it < niter);
-    if (active) {
-      const int rel_qt = nqt - 1 - c_qt;
+  // Role A handles tile `it` in trip `it`, role B tile `it - 1` (B idles in the first trip, A in the
+  // last).  Each role runs its own copy of the loop nest, and the tiles that need no masking get a
+  // loop whose body is unconditional, so the accumulators are updated in place (a tile body behind a
+  // branch costs a register-to-register copy of all 64 of them per trip).  Both copies execute
+  // niter + 1 barriers.
+  auto role_loop = [&](auto is_b) {
+    constexpr bool ROLE_B = decltype(is_b)::value;
+    int it = 0, c_st = 0, c_par = 0;  // trip, ring stage and mailbox parity of the tile being consumed
+    auto begin_trip = [&]() {
+      feeding = it + 1 < niter;
+      if (feeding) prep();
+    };
+    auto end_trip = [&]() {
+      Loader::wait_all();
+      __syncthreads();
+      it++;
+    };
+    auto idle_trip = [&]() {
+      begin_trip();
+#pragma unroll
+      for (int k = 0; k < kParts; k++) part(k);
+      end_trip();
+    };
+    auto body = [&](auto masked_tag, int rel_qt) {
+      constexpr bool MASKED = decltype(masked_tag)::value;
       const int q0 = (qt0 + rel_qt) * BM;
       lds_cptr Qs = ring + c_st * 2 * BM * HD;
       lds_cptr dOs = Qs + BM * HD;
       MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * 4 * 64 + lane;
       MODA_LDS const float* st_s = stat + c_st * 2 * BM;
-      if (rel_qt >= first_free_qt) {
-        if (!role_b)
-          tile_a(std::false_type{}, Qs, dOs, st_s, mb, q0);
-        else
-          tile_b(Qs, dOs, st_s + BM, mb);
-      } else {
-        const bool touches = (qhi > q0) && (qlo < q0 + BM) && (qhi > qlo);
-        if (__any(touches)) {
-          if (!role_b)
-            tile_a(std::true_type{}, Qs, dOs, st_s, mb, q0);
-          else
-            tile_b(Qs, dOs, st_s + BM, mb);
+      bool run = true;
+      if (MASKED) {
+        run = __any((qhi > q0) && (qlo < q0 + BM) && (qhi > qlo));
+        if (!run) {
+#pragma unroll
+          for (int k = 0; k < kParts; k++) part(k);
         }
       }
-      if (++c_qt == nqt) c_qt = 0;
+      if (run) {
+        if constexpr (ROLE_B)
+          tile_b(Qs, dOs, st_s + BM, mb);
+        else
+          tile_a(MASKED, Qs, dOs, st_s, mb, q0);
+      }
       c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
       c_par ^= 1;
+    };
+    if (ROLE_B) idle_trip();
+    for (int gh = 0; gh < a.hdiv; gh++) {
+      int rel_qt = nqt - 1;
+      for (; rel_qt >= first_free_qt; rel_qt--) {
+        begin_trip();
+        body(std::false_type{}, rel_qt);
+        end_trip();
+      }
+      for (; rel_qt >= 0; rel_qt--) {
+        begin_trip();
+        body(std::true_type{}, rel_qt);
+        end_trip();
+      }
     }
-    ld.wait_all();
-    __syncthreads();
-  }
+    if (!ROLE_B) idle_trip();
+  };
+  if (!role_b)
+    role_loop(std::false_type{});
+  else
+    role_loop(std::true_type{});
 
   if (valid) {
     uint16_t* outp;

@@ -161,10 +161,17 @@ struct OperandAddr {
 // flight ahead of the matrix pipe and pin that order with scheduling barriers.
 // Consecutive MFMAs always target different accumulators.
 
+// Every helper takes an optional hook, called as hook(j) right after the j-th MFMA has been issued
+// (j is a constant after unrolling): a place to slip other instructions -- the next tile's
+// global -> LDS loads -- into the stream at a fixed position.
+struct NoHook {
+  __device__ __forceinline__ void operator()(int) const {}
+};
+
 // acc[bb] = sum_kk rows(tile, 32*bb + n, kk) x breg[kk]   (accumulators start at zero)
-template <typename T, int HD, int NB, int DEPTH>
+template <typename T, int HD, int NB, int DEPTH, typename Hook = NoHook>
 __device__ __forceinline__ void mfma_rows(const OperandAddr<HD>& oa, lds_cptr tile, const i32x4 (&breg)[HD / 16],
-                                          f32x16 (&acc)[NB]) {
+                                          f32x16 (&acc)[NB], Hook&& hook = Hook{}) {
   constexpr int KK = HD / 16, N = NB * KK;
   i32x4 ops[N];
 #pragma unroll
@@ -183,13 +190,14 @@ __device__ __forceinline__ void mfma_rows(const OperandAddr<HD>& oa, lds_cptr ti
       acc[bb] = mfma32<T>(ops[j], breg[kk], acc[bb]);
     }
     __builtin_amdgcn_sched_barrier(0);
+    hook(j);
   }
 }
 
 // acc[bb] += sum_kk rows(tile, 32*bb + n, kk) x breg[kk]   (accumulators preset by the caller)
-template <typename T, int HD, int NB, int DEPTH>
+template <typename T, int HD, int NB, int DEPTH, typename Hook = NoHook>
 __device__ __forceinline__ void mfma_rows_acc(const OperandAddr<HD>& oa, lds_cptr tile, const i32x4 (&breg)[HD / 16],
-                                              f32x16 (&acc)[NB]) {
+                                              f32x16 (&acc)[NB], Hook&& hook = Hook{}) {
   constexpr int KK = HD / 16, N = NB * KK;
   i32x4 ops[N];
 #pragma unroll
@@ -200,15 +208,16 @@ __device__ __forceinline__ void mfma_rows_acc(const OperandAddr<HD>& oa, lds_cpt
     if (j + DEPTH < N) ops[j + DEPTH] = oa.row_operand(tile, 32 * ((j + DEPTH) % NB), (j + DEPTH) / NB);
     acc[j % NB] = mfma32<T>(ops[j], breg[j / NB], acc[j % NB]);
     __builtin_amdgcn_sched_barrier(0);
+    hook(j);
   }
 }
 
 // Two tiles against two register operands in one pipeline:
 // acc0[bb] = rows(tile0) x breg0, acc1[bb] = rows(tile1) x breg1.
-template <typename T, int HD, int NB, int DEPTH>
+template <typename T, int HD, int NB, int DEPTH, typename Hook = NoHook>
 __device__ __forceinline__ void mfma_rows2(const OperandAddr<HD>& oa, lds_cptr tile0, const i32x4 (&breg0)[HD / 16],
                                            f32x16 (&acc0)[NB], lds_cptr tile1, const i32x4 (&breg1)[HD / 16],
-                                           f32x16 (&acc1)[NB]) {
+                                           f32x16 (&acc1)[NB], Hook&& hook = Hook{}) {
   constexpr int KK = HD / 16, N = 2 * NB * KK;
   i32x4 ops[N];
   // step j: which = j & 1, bb = (j >> 1) % NB, kk = (j >> 1) / NB
@@ -231,6 +240,7 @@ __device__ __forceinline__ void mfma_rows2(const OperandAddr<HD>& oa, lds_cptr t
     else
       acc0[bb] = mfma32<T>(ops[j], breg0[kk], kk == 0 ? z : acc0[bb]);
     __builtin_amdgcn_sched_barrier(0);
+    hook(j);
   }
 }
 
@@ -245,14 +255,16 @@ struct TrPipe {
     for (int j = 0; j < DEPTH && j < N; j++) ops[j] = oa.tr_operand(tile, 16 * (j / DB), j % DB);
     __builtin_amdgcn_sched_barrier(0);
   }
+  template <typename Hook = NoHook>
   __device__ __forceinline__ void run(const OperandAddr<HD>& oa, lds_cptr tile, const i32x4 (&breg)[NKS],
-                                      f32x16 (&acc)[DB]) {
+                                      f32x16 (&acc)[DB], Hook&& hook = Hook{}) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < N; j++) {
       if (j + DEPTH < N) ops[j + DEPTH] = oa.tr_operand(tile, 16 * ((j + DEPTH) / DB), (j + DEPTH) % DB);
       acc[j % DB] = mfma32<T>(ops[j], breg[j / DB], acc[j % DB]);
       __builtin_amdgcn_sched_barrier(0);
+      hook(j);
     }
   }
 };
@@ -306,15 +318,26 @@ struct TileLoader {
 template <int BYTES>
 __device__ __forceinline__ void lds_dma(i32x4 rsrc, uint32_t lds_byte_addr, int voff, int soff) {
   static_assert(BYTES == 16 || BYTES == 4, "dwordx4 or dword");
+  // The scalar operands are wave-uniform by contract.  Under scalar-register pressure the compiler may
+  // park such a value in a vector register and would then hand that register to the "s" operands
+  // below; reading it back through readfirstlane (free when the value already sits in a scalar
+  // register) keeps the operands legal.
+  const uint32_t m0v = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_byte_addr);
+  const int so = __builtin_amdgcn_readfirstlane(soff);
+  i32x4 rs;
+  rs[0] = __builtin_amdgcn_readfirstlane(rsrc[0]);
+  rs[1] = __builtin_amdgcn_readfirstlane(rsrc[1]);
+  rs[2] = __builtin_amdgcn_readfirstlane(rsrc[2]);
+  rs[3] = __builtin_amdgcn_readfirstlane(rsrc[3]);
   if (BYTES == 16)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
-                 : "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
                  : "memory", "m0");
   else
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
-                 : "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
                  : "memory", "m0");
 }
 
