@@ -113,34 +113,44 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   // loads arriving at once queue up in the CU's address unit and every wave would sit on its issue
   // for hundreds of cycles.  prep() fixes the descriptors of the next tile (wave-uniform, scalar
   // registers only); part(k), k < kParts, issues one load; the tile bodies slip the parts between
-  // the MFMAs of their first phase, early enough for the tile to land within the trip.  Cursor: next tile = (query head ld_gh, query tile ld_qt) into ring stage ld_st.
+  // the MFMAs of their first phase, early enough for the tile to land within the trip.
   constexpr int kParts = 2 * Loader::N + 1;
-  int ld_qt = 0, ld_gh = 0, ld_st = 0;
+  // The cursor is kept as running byte pointers (row f_q0 of the current query head in Q, dO and this
+  // wave's statistic) that step down one tile per call: the scalar unit then has a few adds per trip
+  // instead of a dozen dependent 64-bit multiplies.
+  const uint32_t q_row_bytes = (uint32_t)a.sq.t * 2u, do_row_bytes = (uint32_t)a.sdo.t * 2u;
+  const int voff_q = ld.row_in_pass * (int)q_row_bytes + ld.gchunk * 16;
+  const int voff_do = ld.row_in_pass * (int)do_row_bytes + ld.gchunk * 16;
+  // wave 0 fetches lse ([B, Tq, Hq]: one dword every Hq), wave 1 delta ([B, Hq, Tq]: contiguous)
+  const int voff_stat = wave == 0 ? lane * a.Hq * 4 : lane * 4;
+  const uint32_t stat_row_bytes = wave == 0 ? (uint32_t)a.Hq * 4u : 4u;
+  const char *q_ptr = nullptr, *do_ptr = nullptr, *st_ptr = nullptr;
+  int f_q0 = 0, f_left = 0, ld_gh = 0, ld_st = 0;
+  auto seek_head = [&]() {  // top tile of query head ld_gh
+    const int hq = hkv * a.hdiv + ld_gh;
+    f_q0 = (qt0 + nqt - 1) * BM;
+    f_left = nqt;
+    q_ptr = (const char*)(a.q + b * a.sq.b + hq * a.sq.h + (int64_t)f_q0 * a.sq.t);
+    do_ptr = (const char*)(a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)f_q0 * a.sdo.t);
+    st_ptr = wave == 0 ? (const char*)(a.lse + ((int64_t)b * a.Tq + f_q0) * a.Hq + hq)
+                       : (const char*)(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + f_q0);
+    ld_gh++;
+  };
   i32x4 rs_q, rs_do, rs_stat;
   uint32_t lds_q, lds_stat;
-  int voff_q, voff_do, voff_stat;
   auto prep = [&]() {
-    const int q0 = (qt0 + nqt - 1 - ld_qt) * BM;  // tiles are walked from the last one down
-    const int hq = hkv * a.hdiv + ld_gh;
-    const int rows = max(min(a.Tq - q0, BM), 0);
-    rs_q = rsrc_words(a.q + b * a.sq.b + hq * a.sq.h + (int64_t)q0 * a.sq.t, (uint32_t)rows * (uint32_t)a.sq.t * 2u);
-    rs_do = rsrc_words(a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)q0 * a.sdo.t, (uint32_t)rows * (uint32_t)a.sdo.t * 2u);
-    voff_q = ld.row_in_pass * (int)a.sq.t * 2 + ld.gchunk * 16;
-    voff_do = ld.row_in_pass * (int)a.sdo.t * 2 + ld.gchunk * 16;
+    if (f_left == 0) seek_head();
+    const uint32_t rows = (uint32_t)max(min(a.Tq - f_q0, BM), 0);  // only a head's top tile can be short
+    rs_q = rsrc_words(q_ptr, rows * q_row_bytes);
+    rs_do = rsrc_words(do_ptr, rows * do_row_bytes);
+    rs_stat = rsrc_words(st_ptr, rows > 0 ? (rows - 1) * stat_row_bytes + 4u : 0u);
     lds_q = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr(ring + ld_st * 2 * BM * HD + wave * 512));
-    // per-row statistics straight into LDS as well: wave 0 fetches lse, wave 1 delta (one dword per lane)
-    if (wave == 0) {
-      rs_stat = rsrc_words(a.lse + ((int64_t)b * a.Tq + q0) * a.Hq + hq, rows > 0 ? ((rows - 1) * a.Hq + 1) * 4u : 0u);
-      voff_stat = lane * a.Hq * 4;
-    } else {
-      rs_stat = rsrc_words(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + q0, (uint32_t)rows * 4u);
-      voff_stat = lane * 4;
-    }
     lds_stat = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(stat + ld_st * 2 * BM + (wave == 0 ? 0 : BM)));
-    if (++ld_qt == nqt) {
-      ld_qt = 0;
-      ld_gh++;
-    }
+    q_ptr -= (int64_t)BM * q_row_bytes;
+    do_ptr -= (int64_t)BM * do_row_bytes;
+    st_ptr -= (int64_t)BM * stat_row_bytes;
+    f_q0 -= BM;
+    f_left--;
     ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
   };
   bool feeding = false;  // this trip has a tile to fetch
@@ -148,10 +158,10 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     if (!feeding) return;
     __builtin_amdgcn_sched_barrier(0);
     if (k < Loader::N)
-      lds_dma<16>(rs_q, lds_q + k * 8 * 1024, voff_q, k * 8 * Loader::RPW * (int)a.sq.t * 2);
+      lds_dma<16>(rs_q, lds_q + k * 8 * 1024, voff_q, k * 8 * Loader::RPW * (int)q_row_bytes);
     else if (k < 2 * Loader::N)
       lds_dma<16>(rs_do, lds_q + BM * HD * 2 + (k - Loader::N) * 8 * 1024, voff_do,
-                  (k - Loader::N) * 8 * Loader::RPW * (int)a.sdo.t * 2);
+                  (k - Loader::N) * 8 * Loader::RPW * (int)do_row_bytes);
     else if (wave < 2)
       lds_dma<4>(rs_stat, lds_stat, voff_stat, 0);
     __builtin_amdgcn_sched_barrier(0);
