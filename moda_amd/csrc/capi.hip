@@ -30,6 +30,10 @@ bool aligned(const void* p, const moda_hip_strides& s, int esize) {
   return ((uintptr_t)p % 16 == 0) && (s.b % m == 0) && (s.t % m == 0) && (s.h % m == 0);
 }
 
+// The streaming kernels address rows inside a tile with 32-bit byte offsets: a row stride must stay
+// below 16 MiB (tiles have at most 64 rows per pass).
+bool row_stride_ok(const moda_hip_strides& s, int esize) { return s.t >= 0 && s.t * esize < (1ll << 24); }
+
 bool use_mfma(const moda_hip_desc* d) {
   return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && (d->D == 64 || d->D == 128);
 }
@@ -82,8 +86,9 @@ int check_device() {
 
 #define MODA_REQ_PTR(p) \
   if (!(p)) return MODA_HIP_EINVAL
-#define MODA_REQ_ALIGN(p, s) \
-  if (!aligned((p), (s), es)) return MODA_HIP_EALIGN
+#define MODA_REQ_ALIGN(p, s)                              \
+  if (!aligned((p), (s), es)) return MODA_HIP_EALIGN; \
+  if (!row_stride_ok((s), es)) return MODA_HIP_EUNSUPPORTED
 
 }  // namespace
 

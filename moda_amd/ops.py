@@ -53,6 +53,7 @@ def _usable(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
         and all(x.stride(i) % m == 0 for i in range(3))
         and x.data_ptr() % 16 == 0
         and all(x.stride(i) >= 0 for i in range(3))
+        and x.stride(1) * x.element_size() < (1 << 24)  # row offsets inside a tile are 32-bit
     )
     return x if ok else x.contiguous()
 

@@ -429,6 +429,36 @@ def test_bitwise_determinism(gpu_device):
         assert torch.equal(a[n], b[n]), n
 
 
+def test_slices_wider_than_32bit_offsets(gpu_device):
+    """K/V and depth K/V read in place from views whose (batch, head) slice spans more bytes than a
+    32-bit buffer offset reaches: results must equal those of compact copies bit for bit."""
+    B, T, H, D, L, G = 1, 4096, 1, 64, 2, 2
+    inp = to_dev(oracle.make_inputs(B, T, H, D, L, G, seed=23, dtype=torch.bfloat16, std=0.5), gpu_device)
+    row = 1 << 19  # elements between rows: 1 MiB, so 4096 rows span 4 GiB and the depth rows 8 GiB
+
+    def spread(x):
+        rows = x.shape[1]
+        buf = torch.empty(rows * row, dtype=x.dtype, device=x.device)
+        view = buf.as_strided((B, rows, H, D), (rows * row, row, D, 1))
+        view.copy_(x)
+        return view
+
+    wide = dict(inp)
+    for n in ("k", "v", "kd", "vd"):
+        wide[n] = spread(inp[n])
+        assert wide[n].stride(1) * wide[n].shape[1] * 2 >= (1 << 32)
+    say("CASE wide-slices")
+    a = run_hip(inp, D ** -0.5, G, "causal")
+    b = run_hip(wide, D ** -0.5, G, "causal")
+    for n in a:
+        assert torch.equal(a[n], b[n]), n
+    rows = torch.tensor([0, 1, 4095 * G, T * G - 1])
+    cpu = {k: (None if v is None else v.cpu()) for k, v in inp.items()}
+    ref = oracle.moda_rows_subset(cpu, rows, D ** -0.5, G, "causal")
+    check("o", b["o"][:, rows.to(gpu_device)], ref["o"], torch.bfloat16, "wide-slices")
+    check("dq", b["dq"][:, rows.to(gpu_device)], ref["dq"], torch.bfloat16, "wide-slices")
+
+
 def test_empty_and_degenerate(gpu_device):
     import moda_amd
 
