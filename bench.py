@@ -147,8 +147,21 @@ def bench_reorg(dev, B, T, Hkv, D, L, iters=10):
     ms = s.elapsed_time(e) / iters
     nbytes = 2 * B * T * L * Hkv * D * 2
     gbs = nbytes / (ms * 1e-3) / 1e9
-    return {"kernel": "reorg_kernel", "ms": ms, "bytes": nbytes, "achieved": gbs, "unit": "GB/s",
-            "peak": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS, "bound": "hbm"}
+    out = {"kernel": "reorg_kernel", "ms": ms, "bytes": nbytes, "achieved": gbs, "unit": "GB/s",
+           "peak": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS, "bound": "hbm"}
+    # in-place append of ONE layer into slot L-1 of the preallocated cache (what a layer costs when the
+    # cache is kept and the kernels are given depth_valid, instead of the rebuild above for every layer)
+    for _ in range(2):
+        depth_cache._reorg_fwd(layers[:1], cache, L - 1, L)
+    s.record()
+    for _ in range(iters):
+        depth_cache._reorg_fwd(layers[:1], cache, L - 1, L)
+    e.record()
+    torch.cuda.synchronize()
+    ms1 = s.elapsed_time(e) / iters
+    nb1 = 2 * B * T * Hkv * D * 2
+    out["append_one_layer"] = {"ms": ms1, "bytes": nb1, "achieved": nb1 / (ms1 * 1e-3) / 1e9, "unit": "GB/s"}
+    return out
 
 
 def main():

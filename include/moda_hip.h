@@ -21,6 +21,14 @@
  *   head-dim GQA layout (mode PLAIN_GQA, causal, no depth stream)
  *     q, o, do, dq : [B, T, H*G, D]   query head hq reads kv head hq / G
  *     lse          : [B, T, H*G]
+ *
+ * Partially filled depth stream (no counterpart in the reference, which rebuilds a
+ * compact [B, T*L, H, D] cache for every layer, vision_tasks/deit/models.py:361-390):
+ * with 0 < L_valid < L the depth tensors keep their L slots per token but only
+ * slots l < L_valid are visible; results equal those for the compacted tensors
+ * [B, T*L_valid, H, D], and dkd, dvd are written as zeros in the other slots.
+ * The invisible slots are still read (and multiplied by zero): they must hold
+ * finite values.  Not available with MODA_HIP_CHUNK_VISIBLE.
  */
 #ifndef MODA_HIP_H_
 #define MODA_HIP_H_
@@ -32,7 +40,7 @@
 extern "C" {
 #endif
 
-#define MODA_HIP_VERSION 100
+#define MODA_HIP_VERSION 101
 
 enum moda_hip_dtype { MODA_HIP_BF16 = 0, MODA_HIP_FP16 = 1, MODA_HIP_FP32 = 2 };
 
@@ -64,7 +72,7 @@ typedef struct moda_hip_desc {
   int32_t struct_size;  /* sizeof(moda_hip_desc), checked                         */
   int32_t dtype;        /* moda_hip_dtype of q,k,v,kd,vd,o,do and all gradients    */
   int32_t mode;         /* moda_hip_mode                                           */
-  int32_t reserved;
+  int32_t L_valid;      /* depth slots per token that hold data; 0 = all L (see below)          */
   int64_t B;            /* batch                                                   */
   int64_t T;            /* tokens (key rows)                                       */
   int64_t H;            /* kv heads                                                */

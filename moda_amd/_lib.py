@@ -38,7 +38,7 @@ class Desc(Structure):
         ("struct_size", c_int32),
         ("dtype", c_int32),
         ("mode", c_int32),
-        ("reserved", c_int32),
+        ("L_valid", c_int32),
         ("B", c_int64),
         ("T", c_int64),
         ("H", c_int64),

@@ -64,6 +64,8 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   const int c_first = (dep ? ct - n_seq_tiles : ct) * BN;
   const int c = c_first + kblk * 32 + n;
   const bool valid = c < ncols;
+  // a depth slot without data: no row sees it; its K/V are replaced by zeros, its gradients come out zero
+  const bool empty_slot = dep && valid && (c % a.L) >= a.Lv;
 
   // stationary operand of this wave's role: K rows (A) or V rows (B)
   i32x4 Sr[KK];
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       i32x4 z = {0, 0, 0, 0};
-      Sr[kk] = valid ? *reinterpret_cast<const i32x4*>(src + (int64_t)c * st + 16 * kk + 8 * g) : z;
+      Sr[kk] = (valid && !empty_slot) ? *reinterpret_cast<const i32x4*>(src + (int64_t)c * st + 16 * kk + 8 * g) : z;
     }
   }
 
@@ -97,7 +99,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     }
   };
   int qlo = 0, qhi = 0;
-  if (valid) q_interval(c, qlo, qhi);
+  if (valid && !empty_slot) q_interval(c, qlo, qhi);
   int wg_lo, wg_hi, tmp;
   q_interval(c_first, wg_lo, tmp);
   q_interval(min(ncols, c_first + BN) - 1, tmp, wg_hi);

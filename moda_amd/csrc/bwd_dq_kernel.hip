@@ -86,7 +86,7 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const
     if (a.L > 0) {
       const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
       dlo = lo_t * a.L;
-      dhi = (t + 1) * a.L;
+      dhi = a.chunk ? (t + 1) * a.L : dlo + a.Lv;  // the token's filled slots
     }
   }
   const int r_first = qt * BM;

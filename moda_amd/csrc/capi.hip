@@ -48,6 +48,8 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   if (d->mode == MODA_HIP_PLAIN_GQA && d->L != 0) return MODA_HIP_EINVAL;
   if (d->mode == MODA_HIP_DEPTH_ONLY && d->L == 0) return MODA_HIP_EINVAL;
   if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L > 0 && d->chunk_tokens <= 0) return MODA_HIP_EINVAL;
+  if (d->L_valid < 0 || d->L_valid > d->L) return MODA_HIP_EINVAL;
+  if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L_valid != 0 && d->L_valid != d->L) return MODA_HIP_EUNSUPPORTED;
   // 32-bit index space used for rows and flattened depth columns inside the kernels
   if (d->T * d->G >= (1ll << 30) || d->T * (d->L > 0 ? d->L : 1) >= (1ll << 30) || d->B * d->H * d->G >= (1ll << 20))
     return MODA_HIP_EUNSUPPORTED;
@@ -61,6 +63,7 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   a.Hq = plain ? (int)(d->H * d->G) : (int)d->H;
   a.hdiv = plain ? (int)d->G : 1;
   a.L = (int)d->L;
+  a.Lv = d->L_valid > 0 ? (int)d->L_valid : (int)d->L;
   a.Cb = d->mode == MODA_HIP_CHUNK_VISIBLE ? (int)(d->chunk_tokens > 0 ? d->chunk_tokens : 1) : 1;
   a.has_seq = d->mode != MODA_HIP_DEPTH_ONLY;
   a.causal = d->mode == MODA_HIP_CAUSAL || d->mode == MODA_HIP_CHUNK_VISIBLE || plain;

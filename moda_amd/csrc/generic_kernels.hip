@@ -51,7 +51,7 @@ __device__ __forceinline__ bool row_geom(const KArgs& a, int64_t gid, RowGeom& g
   if (a.L > 0) {
     const int lo_t = a.chunk ? (g.t / a.Cb) * a.Cb : g.t;
     g.dlo = lo_t * a.L;
-    g.dhi = (g.t + 1) * a.L;
+    g.dhi = a.chunk ? (g.t + 1) * a.L : g.dlo + a.Lv;  // the token's filled slots
   }
   return true;
 }
@@ -198,6 +198,7 @@ __global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a, const i
     const int w = col / a.L;
     qlo = w * a.Gf;
     qhi = a.chunk ? min(a.T, (w / a.Cb + 1) * a.Cb) * a.Gf : (w + 1) * a.Gf;
+    if (col - w * a.L >= a.Lv) qhi = qlo;  // a slot without data: no row sees it, its gradients are zero
   }
   float dk[kDR], dv[kDR];
 #pragma unroll

@@ -19,7 +19,8 @@ struct KArgs {
   int Gf;    // query rows per token (fold factor)
   int Hq;    // query-head programs per batch
   int hdiv;  // kv head = hq / hdiv
-  int L;     // depth slots per token
+  int L;     // depth slots per token in the depth tensors (row t*L + l = slot l of token t)
+  int Lv;    // slots per token that hold data, 1 <= Lv <= L: slots l >= Lv are invisible
   int Cb;    // chunk-visible: tokens per chunk
   int has_seq, causal, chunk;
   int nqt;   // query tiles per (batch, query head)

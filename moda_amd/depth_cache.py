@@ -78,15 +78,19 @@ def build_depth_cache(kv_list: Sequence[Tuple[torch.Tensor, torch.Tensor]]):
 
 class DepthCache:
     """Preallocated depth stream: ``append`` writes one layer's K and V into its
-    slot of the token-major buffers; ``view(L)`` returns the ``[B, T*L, H, D]``
-    tensors for the first ``L`` slots when ``L == L_max`` (zero-copy) or a
-    compacted copy otherwise.  Inference/no-grad use only."""
+    slot of the token-major buffers.  ``filled()`` returns ``(k, v, n)``: the whole
+    ``[B, T*L_max, H, D]`` buffers and the number of slots written so far, to be
+    passed as ``cached_k, cached_v, depth_valid=n`` -- nothing is copied or rebuilt
+    between layers (the reference re-stacks all previous layers for every layer,
+    vision_tasks/deit/models.py:383-387).  The buffers start as zeros because the
+    kernels read (and multiply by zero) the unwritten slots.  Inference/no-grad use
+    only: ``append`` writes in place."""
 
     def __init__(self, B: int, T: int, L_max: int, H: int, D: int, dtype, device):
         self.shape = (B, T, H, D)
         self.L_max = L_max
-        self.k = torch.empty(B, T * L_max, H, D, dtype=dtype, device=device)
-        self.v = torch.empty(B, T * L_max, H, D, dtype=dtype, device=device)
+        self.k = torch.zeros(B, T * L_max, H, D, dtype=dtype, device=device)
+        self.v = torch.zeros(B, T * L_max, H, D, dtype=dtype, device=device)
         self.n = 0
 
     def append(self, k: torch.Tensor, v: torch.Tensor):
@@ -94,6 +98,10 @@ class DepthCache:
         _reorg_fwd([k.contiguous()], self.k, self.n, self.L_max)
         _reorg_fwd([v.contiguous()], self.v, self.n, self.L_max)
         self.n += 1
+
+    def filled(self):
+        assert self.n > 0, "depth cache is empty"
+        return self.k, self.v, self.n
 
     def full(self):
         assert self.n == self.L_max

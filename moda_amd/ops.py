@@ -72,7 +72,7 @@ def _check_device(x: torch.Tensor):
 
 
 def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=None, dk=None, dv=None, dkd=None,
-          dvd=None) -> Desc:
+          dvd=None, depth_valid=None) -> Desc:
     d = Desc()
     d.struct_size = ctypes.sizeof(Desc)
     if q.dtype not in _DTYPES:
@@ -85,6 +85,9 @@ def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=
     d.G = G
     d.D = q.shape[3]
     d.L = L
+    if depth_valid is not None and L > 0:
+        assert 1 <= depth_valid <= L, f"depth_valid must be in [1, {L}], got {depth_valid}"
+        d.L_valid = int(depth_valid)
     if mode == _lib.DEPTH_ONLY:
         d.T = q.shape[1] // G
     else:
@@ -108,7 +111,7 @@ def _same_dtype(*xs):
             raise TypeError(f"all tensors must share one dtype, got {dt} and {x.dtype}")
 
 
-def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0):
+def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None):
     """Launch the forward kernels. Returns (o, lse)."""
     _check_device(q)
     _same_dtype(q, k, v, kd, vd)
@@ -125,7 +128,7 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0):
     lse = torch.empty(q.shape[0], q.shape[1], q.shape[2], dtype=torch.float32, device=q.device)
     if L == 0:
         kd = vd = None
-    d = _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=o)
+    d = _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=o, depth_valid=depth_valid)
     with torch.cuda.device(q.device):
         rc = _lib.load().moda_hip_fwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kd), _ptr(vd), _ptr(o),
                                       _ptr(lse), _stream(q))
@@ -133,7 +136,8 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0):
     return o, lse
 
 
-def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages=_lib.STAGE_ALL, out=None, ws=None):
+def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages=_lib.STAGE_ALL, out=None, ws=None,
+             depth_valid=None):
     """Launch the backward kernels. Returns (dq, dk, dv, dkd, dvd).
 
     ``stages`` selects a subset of {delta, dq, dk/dv}; ``out`` (a previous return
@@ -154,7 +158,7 @@ def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages
         dvd = torch.empty(vd.shape, dtype=vd.dtype, device=q.device) if vd is not None else None
     kd_a, vd_a, dkd_a, dvd_a = (kd, vd, dkd, dvd) if L > 0 else (None, None, None, None)
     d = _desc(mode, q, k, v, kd_a, vd_a, G, L, chunk_tokens, scale, o=o, do=do, dq=dq, dk=dk, dv=dv, dkd=dkd_a,
-              dvd=dvd_a)
+              dvd=dvd_a, depth_valid=depth_valid)
     lib = _lib.load()
     nbytes = lib.moda_hip_bwd_workspace_bytes(ctypes.byref(d))
     if ws is None:
@@ -179,8 +183,10 @@ def _assert_group_tile(moda_group_num: int, rows: int = 128):
 
 def parallel_moda_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, cached_v=None, moda_group_num=1,
                       is_causal=True, customized_BT=None, customized_BS=None, customized_BK=None, customized_BV=None,
-                      customized_num_warps=None):
-    """moda_v14.py:381-522.  Returns ``(o, lse)``; tile-size knobs are accepted and ignored."""
+                      customized_num_warps=None, depth_valid=None):
+    """moda_v14.py:381-522.  Returns ``(o, lse)``; tile-size knobs are accepted and ignored.
+    ``depth_valid`` (not in the reference): only the first ``depth_valid`` of the ``L`` slots per token
+    of ``cached_k/v`` are visible."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
     assert cu_seqlens is None, "cu_seqlens is not supported in this version"
     assert q.shape[2] == k.shape[2], (
@@ -190,13 +196,13 @@ def parallel_moda_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, 
     )
     _assert_group_tile(moda_group_num)
     mode = _lib.CAUSAL if is_causal else _lib.NONCAUSAL
-    return _raw_fwd(mode, q, k, v, cached_k, cached_v, scale, moda_group_num)
+    return _raw_fwd(mode, q, k, v, cached_k, cached_v, scale, moda_group_num, depth_valid=depth_valid)
 
 
 def parallel_moda_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None, cached_k=None,
                       cached_v=None, moda_group_num=1, is_causal=True, customized_BT=None, customized_BS=None,
                       customized_BK=None, customized_BV=None, customized_num_warps=None, group_bs=None,
-                      group_warps=None, depth_bs=None, depth_warps=None):
+                      group_warps=None, depth_bs=None, depth_warps=None, depth_valid=None):
     """moda_v14.py:1470-1842.  Returns ``(dq, dk, dv, dg_cumsum=None, d_cached_k, d_cached_v)``."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
     assert cu_seqlens is None, "cu_seqlens is not supported in this version"
@@ -209,7 +215,8 @@ def parallel_moda_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128,
         scale = q.shape[-1] ** -0.5
     _assert_group_tile(moda_group_num)
     mode = _lib.CAUSAL if is_causal else _lib.NONCAUSAL
-    dq, dk, dv, dkd, dvd = _raw_bwd(mode, q, k, v, cached_k, cached_v, o, lse, do, scale, moda_group_num)
+    dq, dk, dv, dkd, dvd = _raw_bwd(mode, q, k, v, cached_k, cached_v, o, lse, do, scale, moda_group_num,
+                                    depth_valid=depth_valid)
     return dq, dk, dv, None, dkd, dvd
 
 
@@ -249,9 +256,9 @@ class ParallelMixtureOfDepthAttentionFunction(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, q, k, v, g, scale, cu_seqlens, cached_k=None, cached_v=None, moda_group_num=1, is_causal=True,
-                group_bs=None, group_warps=None, depth_bs=None, depth_warps=None):
+                group_bs=None, group_warps=None, depth_bs=None, depth_warps=None, depth_valid=None):
         o, lse = _autograd_forward(ctx, parallel_moda_fwd, q, k, v, g, scale, cu_seqlens, cached_k, cached_v,
-                                   moda_group_num, is_causal=is_causal)
+                                   moda_group_num, is_causal=is_causal, depth_valid=depth_valid)
         ctx.mark_non_differentiable(lse)
         return o, lse
 
@@ -259,7 +266,7 @@ class ParallelMixtureOfDepthAttentionFunction(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, do, dlse_unused):
         dq, dk, dv, dkd, dvd = _autograd_backward(ctx, parallel_moda_bwd, do)
-        return dq, dk, dv, None, None, None, dkd, dvd, None, None, None, None, None, None
+        return dq, dk, dv, None, None, None, dkd, dvd, None, None, None, None, None, None, None
 
 
 def _prepare_inputs(api_name, q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first,
@@ -313,21 +320,24 @@ def _prepare_inputs(api_name, q, k, v, g, cached_k, cached_v, scale, moda_group_
 def parallel_moda(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_seqlens=None, moda_group_num=1,
                   is_causal=True, head_first=False, need_lse=False, return_depth_grads=True, warn_shape=True,
                   customized_BT=None, customized_BS=None, customized_BT_backward=None, customized_BS_backward=None,
-                  group_bs=None, group_warps=None, depth_bs=None, depth_warps=None):
-    """Fused sequence+depth attention; signature of moda_v14.py:2792-2815.
+                  group_bs=None, group_warps=None, depth_bs=None, depth_warps=None, depth_valid=None):
+    """Fused sequence+depth attention; signature of moda_v14.py:2792-2815, plus ``depth_valid``.
 
     q ``[B, T*G, H, D]``; k, v ``[B, T, H, D]``; cached_k/v ``[B, T*L, H, D]`` or
     None.  Returns ``o`` (q.dtype) or ``(o, lse)`` with ``lse`` fp32 in base-2
     units.  The ``customized_*``, ``group_*`` and ``depth_*`` knobs tune the
     reference's Triton launches and have no meaning here; they are accepted and
-    ignored.
+    ignored.  ``depth_valid`` (an extension): ``cached_k/v`` keep ``L`` slots per token
+    but only the first ``depth_valid`` are visible -- the result equals that for the
+    compacted ``[B, T*depth_valid, H, D]`` tensors, the gradients of the other slots are
+    zero, and a preallocated cache (``DepthCache``) need not be rebuilt per layer.
     """
     q, k, v, g, cached_k, cached_v, scale = _prepare_inputs(
         "parallel_moda", q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first, return_depth_grads,
         warn_shape)
     o, lse = ParallelMixtureOfDepthAttentionFunction.apply(
         q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, is_causal, group_bs, group_warps, depth_bs,
-        depth_warps)
+        depth_warps, depth_valid)
     return (o, lse) if need_lse else o
 
 

@@ -15,6 +15,8 @@ from .moda_oracle import (  # noqa: F401
     plain_gqa_dense,
     depth_cache_ref,
     depth_cache_grad_ref,
+    compact_depth,
+    scatter_depth_grad,
     make_inputs,
     error_metrics,
     passes_reference_rule,

@@ -235,6 +235,30 @@ def moda_rows_subset(inp, rows: torch.Tensor, scale, G, mode, chunk_tokens=0, dt
 
 
 # --------------------------------------------------------------------------
+# partially filled depth stream (an extension of this build; no reference counterpart)
+# --------------------------------------------------------------------------
+def compact_depth(x: torch.Tensor, T: int, valid: int) -> torch.Tensor:
+    """``[B, T*L, H, D]`` -> ``[B, T*valid, H, D]`` keeping slots ``l < valid`` of every token.
+
+    This DEFINES the ``depth_valid`` option of the kernels: with ``depth_valid = valid`` they must
+    return what the functions of this file return for the compacted tensors (the layout is that of
+    vision_tasks/deit/models.py:361-375: row ``t*L + l`` = slot ``l`` of token ``t``)."""
+    B, TL, H, D = x.shape
+    L = TL // T
+    return x.reshape(B, T, L, H, D)[:, :, :valid].reshape(B, T * valid, H, D)
+
+
+def scatter_depth_grad(g: torch.Tensor, T: int, L: int) -> torch.Tensor:
+    """Gradient w.r.t. the compacted depth tensor -> gradient w.r.t. the ``L``-slot tensor (zeros in
+    the slots that were dropped)."""
+    B, TV, H, D = g.shape
+    valid = TV // T
+    out = torch.zeros(B, T, L, H, D, dtype=g.dtype, device=g.device)
+    out[:, :, :valid] = g.reshape(B, T, valid, H, D)
+    return out.reshape(B, T * L, H, D)
+
+
+# --------------------------------------------------------------------------
 # (iii) blockwise evaluation with explicit gradient formulas
 # --------------------------------------------------------------------------
 @torch.no_grad()

@@ -32,7 +32,7 @@ def test_descriptor_layout_and_version():
     from moda_amd import _lib
 
     lib = _lib.load()
-    assert lib.moda_hip_version() == 100
+    assert lib.moda_hip_version() == 101
     assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24
     assert _lib.Desc.q.offset == 80
     # a descriptor with the wrong struct_size is rejected without touching any device

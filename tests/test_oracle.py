@@ -263,3 +263,21 @@ def test_golden_fixture_matches_oracle():
                 assert key not in z
             else:
                 assert np.allclose(z[key], r[n].numpy(), atol=1e-6), key
+
+
+def test_compact_and_scatter_depth_are_adjoint_slot_selections():
+    """compact_depth keeps exactly rows t*L + l with l < valid, in order; scatter_depth_grad is its
+    transpose (checked against autograd and against a literal index loop)."""
+    B, T, L, H, D, valid = 2, 5, 4, 3, 2, 3
+    x = torch.arange(B * T * L * H * D, dtype=torch.float64).reshape(B, T * L, H, D).requires_grad_(True)
+    c = oracle.compact_depth(x, T, valid)
+    assert c.shape == (B, T * valid, H, D)
+    for t in range(T):
+        for l in range(valid):
+            assert torch.equal(c[:, t * valid + l], x[:, t * L + l])
+    w = torch.randn_like(c)
+    (c * w).sum().backward()
+    assert torch.equal(x.grad, oracle.scatter_depth_grad(w, T, L))
+    for t in range(T):
+        for l in range(valid, L):
+            assert x.grad[:, t * L + l].abs().max() == 0

@@ -459,6 +459,71 @@ def test_slices_wider_than_32bit_offsets(gpu_device):
     check("dq", b["dq"][:, rows.to(gpu_device)], ref["dq"], torch.bfloat16, "wide-slices")
 
 
+@pytest.mark.parametrize("case", [
+    # (B, T, H, D, L, valid, G, mode, dtype)
+    (2, 150, 2, 64, 5, 3, 2, "causal", torch.bfloat16),
+    (1, 333, 2, 128, 6, 1, 4, "causal", torch.bfloat16),
+    (2, 197, 3, 64, 12, 7, 1, "noncausal", torch.float16),
+    (2, 97, 2, 128, 4, 4, 1, "causal", torch.bfloat16),
+    (2, 130, 2, 64, 9, 2, 2, "depth_only", torch.bfloat16),
+    (1, 70, 2, 96, 5, 2, 2, "causal", torch.bfloat16),   # generic kernels (head dim 96)
+    (1, 60, 2, 64, 3, 2, 1, "causal", torch.float32),    # generic kernels (fp32)
+])
+def test_partially_filled_depth_stream(gpu_device, case):
+    """depth_valid = v on the L-slot tensors == the compacted [B, T*v, H, D] tensors (the oracle's
+    definition); the unused slots hold large finite junk and must get exactly zero gradient."""
+    from moda_amd import ops
+
+    B, T, H, D, L, valid, G, mode, dtype = case
+    say(f"CASE partial-depth {case}")
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=29, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
+    junk = torch.Generator().manual_seed(5)
+    for n in ("kd", "vd"):
+        x = inp[n].reshape(B, T, L, H, D)
+        x[:, :, valid:] = (30.0 * torch.randn(x[:, :, valid:].shape, generator=junk)).to(dtype)
+    comp = dict(inp)
+    comp["kd"] = oracle.compact_depth(inp["kd"], T, valid).contiguous()
+    comp["vd"] = oracle.compact_depth(inp["vd"], T, valid).contiguous()
+    scale = D ** -0.5
+    ref = oracle.moda_dense_fwd_bwd(comp, scale, G, mode, 0)
+    ref["dkd"] = oracle.scatter_depth_grad(ref["dkd"], T, L)
+    ref["dvd"] = oracle.scatter_depth_grad(ref["dvd"], T, L)
+    dev = to_dev(inp, gpu_device)
+    m = MODE_ID[mode]
+    o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], scale, G, 0, depth_valid=valid)
+    dq, dk, dv, dkd, dvd = ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], o, lse, dev["do"], scale,
+                                        G, 0, depth_valid=valid)
+    got = {"o": o, "lse": lse, "dq": dq, "dk": dk, "dv": dv, "dkd": dkd, "dvd": dvd}
+    compare_all(got, ref, dtype, f"partial-depth {case}")
+    for n in ("dkd", "dvd"):
+        unused = got[n].reshape(B, T, L, H, D)[:, :, valid:]
+        assert unused.numel() == 0 or unused.float().abs().max().item() == 0.0, n
+
+
+def test_depth_cache_append_in_place(gpu_device):
+    """DepthCache.append + depth_valid reproduces, layer by layer, what the rebuilt compact cache gives
+    (vision_tasks/deit/models.py:383-387 rebuilds it for every layer)."""
+    import moda_amd
+
+    B, T, H, D, Lmax, G = 2, 64, 2, 64, 4, 2
+    gen = torch.Generator().manual_seed(31)
+    q = (0.5 * torch.randn(B, T * G, H, D, generator=gen)).bfloat16().to(gpu_device)
+    k = (0.5 * torch.randn(B, T, H, D, generator=gen)).bfloat16().to(gpu_device)
+    v = (0.5 * torch.randn(B, T, H, D, generator=gen)).bfloat16().to(gpu_device)
+    layers = [((0.5 * torch.randn(B, T, H, D, generator=gen)).bfloat16().to(gpu_device),
+               (0.5 * torch.randn(B, T, H, D, generator=gen)).bfloat16().to(gpu_device)) for _ in range(Lmax)]
+    cache = moda_amd.DepthCache(B, T, Lmax, H, D, torch.bfloat16, gpu_device)
+    for n in range(1, Lmax + 1):
+        cache.append(*layers[n - 1])
+        ck, cv, nv = cache.filled()
+        assert nv == n
+        with torch.no_grad():
+            o_inplace = moda_amd.parallel_moda(q, k, v, cached_k=ck, cached_v=cv, moda_group_num=G, depth_valid=nv)
+            rk, rv = moda_amd.build_depth_cache(layers[:n])
+            o_rebuilt = moda_amd.parallel_moda(q, k, v, cached_k=rk, cached_v=rv, moda_group_num=G)
+        assert (o_inplace.float() - o_rebuilt.float()).abs().max().item() <= 2.0 ** -6, n
+
+
 def test_empty_and_degenerate(gpu_device):
     import moda_amd
 
