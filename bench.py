@@ -164,6 +164,47 @@ def bench_reorg(dev, B, T, Hkv, D, L, iters=10):
     return out
 
 
+def bench_mfma_probe(dev):
+    """Sustained rate of a pure bf16 MFMA loop on this device, with operands drawn like the workload's
+    inputs (0.5 * N(0,1), bf16) and with zeros.  The matrix pipe is power limited: random operands run
+    at a lower clock than zeros, and well below the published peak, so the attention kernels' roofline
+    fraction is also given against this measured ceiling."""
+    import ctypes
+
+    import torch
+
+    from moda_amd import _lib
+
+    lib = _lib.load()
+    ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    gen = torch.Generator().manual_seed(0)
+    out = {}
+    for name, tab in (("random", (0.5 * torch.randn(512 * 8, generator=gen)).bfloat16()),
+                      ("zeros", torch.zeros(512 * 8, dtype=torch.bfloat16))):
+        tab = tab.to(dev)
+        iters = 200000  # about 30 ms: long enough for the clock to settle
+        stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+        def launch(n):
+            rc = lib.moda_hip_mfma_probe(ctypes.c_void_p(tab.data_ptr()), n, ncu, ctypes.c_void_p(clocks.data_ptr()),
+                                         ctypes.c_void_p(sink.data_ptr()), stream)
+            _lib.check(rc, "moda_hip_mfma_probe")
+
+        launch(20000)
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        launch(iters)
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e)
+        flop = float(ncu) * 8 * iters * 4 * 32768
+        c = clocks.cpu().tolist()
+        out[name] = {"tflops": flop / (ms * 1e-3) / 1e12, "shader_clock_mhz": c[0] / (c[1] / 100.0) if c[1] else None}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -301,6 +342,9 @@ def main():
                                     "moda_over_twin": value / tw_value}
     if L > 0:
         out["depth_reorg"] = bench_reorg(dev, B, T, Hkv, D, L)
+    probe = bench_mfma_probe(dev)
+    out["mfma_probe"] = probe
+    out["frac_of_measured_mfma_rate"] = value / probe["random"]["tflops"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, T, Hkv, G, D, L, mode, cb)
     print(json.dumps(out))

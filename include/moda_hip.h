@@ -158,6 +158,19 @@ int moda_hip_depth_reorg_bwd(const void* d_cache, int64_t n_layers, int64_t slot
                              int64_t B, int64_t T, int64_t H, int64_t D, int32_t dtype,
                              void* const* d_layers, void* stream);
 
+/*
+ * Diagnostic, no counterpart in the reference: runs `iters` rounds of four independent bf16 MFMAs
+ * per wave (eight waves per workgroup, `workgroups` workgroups; 32768 FLOP per MFMA) on the register
+ * operands found in `operands` (device memory, 512 x 16 bytes: lane l of operand j reads entry
+ * 64*j + l; entries 0..255 feed the A side, 256..511 the B side).  The matrix pipe of this GPU is
+ * power limited and its sustained rate depends on the operand bits, so benchmarks time this call
+ * with the same kind of data next to the attention kernels.  `clocks` (device, two uint64, may be
+ * NULL) receives the loop's duration in shader-clock cycles and in 100 MHz ticks.  `sink` is 4 bytes
+ * of device scratch.
+ */
+int moda_hip_mfma_probe(const void* operands, int64_t iters, int64_t workgroups, uint64_t* clocks, float* sink,
+                        void* stream);
+
 /* Human-readable text for an error code (static storage). */
 const char* moda_hip_strerror(int code);
 

@@ -26,6 +26,7 @@ EXPORTS = (
     "moda_hip_depth_reorg_bwd",
     "moda_hip_strerror",
     "moda_hip_version",
+    "moda_hip_mfma_probe",
 )
 
 
@@ -98,6 +99,8 @@ def load():
                                              c_int32, POINTER(vp), vp]
     lib.moda_hip_strerror.restype = c_char_p
     lib.moda_hip_strerror.argtypes = [c_int]
+    lib.moda_hip_mfma_probe.restype = c_int
+    lib.moda_hip_mfma_probe.argtypes = [vp, c_int64, c_int64, vp, vp, vp]
     lib.moda_hip_version.restype = c_int
     lib.moda_hip_version.argtypes = []
     _lib = lib

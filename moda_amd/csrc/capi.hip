@@ -10,6 +10,8 @@ namespace moda {
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream);
+hipError_t launch_mfma_probe(const void* operands, int64_t iters, uint64_t* clocks, float* sink, int blocks,
+                             hipStream_t stream);
 hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_generic(const KArgs& a, int dtype, int D, int which, hipStream_t stream);
 hipError_t launch_reorg(void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t n_tokens,
@@ -266,6 +268,16 @@ int moda_hip_depth_reorg_bwd(const void* d_cache, int64_t n_layers, int64_t slot
   if (B * T >= (1ll << 31)) return MODA_HIP_EUNSUPPORTED;
   hipError_t e = moda::launch_reorg(d_layers, n_layers, slot0, L_total, B * T, H * D * elem_size(dtype),
                                     const_cast<void*>(d_cache), false, (hipStream_t)stream);
+  return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
+}
+
+int moda_hip_mfma_probe(const void* operands, int64_t iters, int64_t workgroups, uint64_t* clocks, float* sink,
+                        void* stream) {
+  if (!operands || !sink || iters < 0 || workgroups <= 0 || workgroups > (1 << 20)) return MODA_HIP_EINVAL;
+  if ((uintptr_t)operands % 16 != 0) return MODA_HIP_EALIGN;
+  int rc = check_device();
+  if (rc) return rc;
+  hipError_t e = moda::launch_mfma_probe(operands, iters, clocks, sink, (int)workgroups, (hipStream_t)stream);
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }
 

@@ -524,6 +524,26 @@ def test_depth_cache_append_in_place(gpu_device):
         assert (o_inplace.float() - o_rebuilt.float()).abs().max().item() <= 2.0 ** -6, n
 
 
+def test_mfma_probe_runs(gpu_device):
+    """The diagnostic entry point launches, finishes and reports both clocks."""
+    import ctypes
+
+    from moda_amd import _lib
+
+    lib = _lib.load()
+    tab = (0.5 * torch.randn(512 * 8)).bfloat16().to(gpu_device)
+    clocks = torch.zeros(2, dtype=torch.int64, device=gpu_device)
+    sink = torch.zeros(1, device=gpu_device)
+    rc = lib.moda_hip_mfma_probe(ctypes.c_void_p(tab.data_ptr()), 1000, 8, ctypes.c_void_p(clocks.data_ptr()),
+                                 ctypes.c_void_p(sink.data_ptr()),
+                                 ctypes.c_void_p(torch.cuda.current_stream(gpu_device).cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    c = clocks.cpu().tolist()
+    assert c[0] >= 1000 * 4 * 16 and c[1] > 0  # at least 16 cycles per MFMA on the shader clock
+    assert lib.moda_hip_mfma_probe(None, 1, 1, None, ctypes.c_void_p(sink.data_ptr()), None) == -1  # MODA_HIP_EINVAL
+
+
 def test_empty_and_degenerate(gpu_device):
     import moda_amd
 
