@@ -166,7 +166,7 @@ def test_golden_fixture(gpu_device):
 
 
 # ---------------------------------------------------------------------------
-# BASELINE configurations
+# the five benchmark configurations (c1 .. c5)
 # ---------------------------------------------------------------------------
 def test_config_c1_fp32(gpu_device):
     """B1 T256 H4 D64 L4 fp32, q pre-scaled by D**-0.5 and scale=1 -- on the GPU in fp32."""
