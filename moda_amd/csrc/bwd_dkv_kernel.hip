@@ -360,13 +360,9 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 template <typename T, int HD>
 hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = 3 * 2 * 64 * HD * sizeof(uint16_t) + 2 * 4 * 4 * 64 * 16 + 3 * 2 * 64 * sizeof(float);
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dkv_kernel<T, HD>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return e;
-    attr_done = true;
-  }
+  static LdsAttrState attr;
+  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_kernel<T, HD>), smem);
+  if (ea != hipSuccess) return ea;
   const int64_t n_seq_tiles = a.has_seq ? (a.T + 127) / 128 : 0;
   const int64_t n_dep_tiles = a.L > 0 ? ((int64_t)a.T * a.L + 127) / 128 : 0;
   const int64_t nblk = (n_seq_tiles + n_dep_tiles) * a.B * a.Hkv;

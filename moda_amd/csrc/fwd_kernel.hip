@@ -238,13 +238,9 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void fwd_kernel(cons
 template <typename T, int HD>
 hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = (size_t)kRowStages * 2 * 64 * HD * sizeof(uint16_t);
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<T, HD>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return e;
-    attr_done = true;
-  }
+  static LdsAttrState attr;
+  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD>), smem);
+  if (ea != hipSuccess) return ea;
   const int64_t nblk = (int64_t)((a.Tq + kRowBM - 1) / kRowBM) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
   hipLaunchKernelGGL((fwd_kernel<T, HD>), dim3((unsigned)nblk), dim3(64 * kRowWaves), smem, stream, a);

@@ -3,6 +3,8 @@
 // and its two read patterns (row operand, transposed operand).
 #pragma once
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 namespace moda {
@@ -268,6 +270,24 @@ struct TrPipe {
     }
   }
 };
+
+// Host side: raise a kernel's dynamic-LDS limit, once per device (the attribute belongs to the device's
+// copy of the kernel, so a process that drives several GPUs needs it on each of them).  `state` is a
+// static of the calling launcher, one per kernel instantiation.
+struct LdsAttrState {
+  std::atomic<uint64_t> devices{0};
+};
+inline hipError_t allow_dynamic_lds(LdsAttrState& state, const void* kernel, size_t bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const bool tracked = dev >= 0 && dev < 64;
+  const uint64_t bit = tracked ? (1ull << dev) : 0;
+  if (tracked && (state.devices.load(std::memory_order_acquire) & bit)) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e == hipSuccess && tracked) state.devices.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 // Raw buffer resource over `nbytes` bytes at `base` (wave-uniform): loads past the end return zero.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t nbytes) {
