@@ -38,9 +38,9 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a) {
   if (r < a.Tq && (tid % TPR) == 0) a.delta[((int64_t)b * a.Hq + hq) * a.Tq + r] = -acc;
 }
 
-template <typename T, int HD>
-__global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void dq_kernel(const KArgs a) {
-  constexpr int BM = kRowBM, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * kRowWaves, NST = kRowStages, DIST = kRowDist;
+template <typename T, int HD, typename Shape>
+__global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a) {
+  constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST, DIST = Shape::DIST;
   static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
@@ -226,22 +226,32 @@ hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <typename T, int HD>
-hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = (size_t)kRowStages * 2 * 64 * HD * sizeof(uint16_t);
+template <typename T, int HD, typename Shape>
+hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
+  constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
   static LdsAttrState attr;
-  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dq_kernel<T, HD>), smem);
+  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dq_kernel<T, HD, Shape>), smem);
   if (ea != hipSuccess) return ea;
-  const int64_t nblk = (int64_t)((a.Tq + kRowBM - 1) / kRowBM) * a.B * a.Hq;
+  const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((dq_kernel<T, HD>), dim3((unsigned)nblk), dim3(64 * kRowWaves), smem, stream, a);
+  hipLaunchKernelGGL((dq_kernel<T, HD, Shape>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
   return hipGetLastError();
 }
 
-template __global__ void dq_kernel<BF16, 128>(const KArgs);
-template __global__ void dq_kernel<BF16, 64>(const KArgs);
-template __global__ void dq_kernel<FP16, 128>(const KArgs);
-template __global__ void dq_kernel<FP16, 64>(const KArgs);
+template <typename T, int HD>
+hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
+  if (use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units)) return launch_dq_t_shape<T, HD, RowSmall<HD>>(a, stream);
+  return launch_dq_t_shape<T, HD, RowLarge>(a, stream);
+}
+
+template __global__ void dq_kernel<BF16, 128, RowLarge>(const KArgs);
+template __global__ void dq_kernel<BF16, 64, RowLarge>(const KArgs);
+template __global__ void dq_kernel<FP16, 128, RowLarge>(const KArgs);
+template __global__ void dq_kernel<FP16, 64, RowLarge>(const KArgs);
+template __global__ void dq_kernel<BF16, 128, RowSmall<128>>(const KArgs);
+template __global__ void dq_kernel<BF16, 64, RowSmall<64>>(const KArgs);
+template __global__ void dq_kernel<FP16, 128, RowSmall<128>>(const KArgs);
+template __global__ void dq_kernel<FP16, 64, RowSmall<64>>(const KArgs);
 
 hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_delta_t<BF16, 128>(a, stream);

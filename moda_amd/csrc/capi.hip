@@ -1,6 +1,8 @@
 // C ABI of libmoda_hip.so (see include/moda_hip.h): descriptor validation and
 // dispatch to the gfx950 kernels.  No tensor-library types cross this file.
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <string.h>
 
 #include "../../include/moda_hip.h"
@@ -75,18 +77,27 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   return MODA_HIP_OK;
 }
 
-int check_device() {
+// The current device must be a gfx950; reports its compute-unit count.  One entry per device is cached.
+int check_device(int* compute_units = nullptr) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return MODA_HIP_EDEVICE;
-  static int cached_dev = -1;
-  static bool cached_ok = false;
-  if (dev != cached_dev) {
+  struct Entry {
+    std::atomic<int> state{0};  // 0 unknown, 1 gfx950, -1 something else
+    int cus = 0;
+  };
+  static Entry cache[64];
+  Entry local;
+  Entry& e = (dev >= 0 && dev < 64) ? cache[dev] : local;
+  int st = e.state.load(std::memory_order_acquire);
+  if (st == 0) {
     hipDeviceProp_t p;
     if (hipGetDeviceProperties(&p, dev) != hipSuccess) return MODA_HIP_EDEVICE;
-    cached_ok = strncmp(p.gcnArchName, "gfx950", 6) == 0;
-    cached_dev = dev;
+    e.cus = p.multiProcessorCount;
+    st = strncmp(p.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+    e.state.store(st, std::memory_order_release);
   }
-  return cached_ok ? MODA_HIP_OK : MODA_HIP_EDEVICE;
+  if (compute_units) *compute_units = e.cus;
+  return st == 1 ? MODA_HIP_OK : MODA_HIP_EDEVICE;
 }
 
 #define MODA_REQ_PTR(p) \
@@ -123,7 +134,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
     MODA_REQ_ALIGN(kd, d->kd);
     MODA_REQ_ALIGN(vd, d->vd);
   }
-  if ((rc = check_device())) return rc;
+  if ((rc = check_device(&a.compute_units))) return rc;
   a.q = (const uint16_t*)q;
   a.k = (const uint16_t*)k;
   a.v = (const uint16_t*)v;
@@ -200,7 +211,7 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
   } else {
     return MODA_HIP_OK;
   }
-  if ((rc = check_device())) return rc;
+  if ((rc = check_device(&a.compute_units))) return rc;
   a.q = (const uint16_t*)q;
   a.k = (const uint16_t*)k;
   a.v = (const uint16_t*)v;

@@ -22,10 +22,10 @@
 
 namespace moda {
 
-template <typename T, int HD>
-__global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void fwd_kernel(const KArgs a) {
-  constexpr int BM = kRowBM, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * kRowWaves, NST = kRowStages,
-                DIST = kRowDist;
+template <typename T, int HD, typename Shape>
+__global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
+  constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST,
+                DIST = Shape::DIST;
   static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
@@ -235,22 +235,32 @@ __global__ __launch_bounds__(64 * kRowWaves, 8 / kRowWaves) void fwd_kernel(cons
   }
 }
 
-template <typename T, int HD>
-hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = (size_t)kRowStages * 2 * 64 * HD * sizeof(uint16_t);
+template <typename T, int HD, typename Shape>
+hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
+  constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
   static LdsAttrState attr;
-  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD>), smem);
+  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD, Shape>), smem);
   if (ea != hipSuccess) return ea;
-  const int64_t nblk = (int64_t)((a.Tq + kRowBM - 1) / kRowBM) * a.B * a.Hq;
+  const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((fwd_kernel<T, HD>), dim3((unsigned)nblk), dim3(64 * kRowWaves), smem, stream, a);
+  hipLaunchKernelGGL((fwd_kernel<T, HD, Shape>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
   return hipGetLastError();
 }
 
-template __global__ void fwd_kernel<BF16, 128>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64>(const KArgs);
+template <typename T, int HD>
+hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
+  if (use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units)) return launch_fwd_t_shape<T, HD, RowSmall<HD>>(a, stream);
+  return launch_fwd_t_shape<T, HD, RowLarge>(a, stream);
+}
+
+template __global__ void fwd_kernel<BF16, 128, RowLarge>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowLarge>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowLarge>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowLarge>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowSmall<128>>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowSmall<64>>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowSmall<128>>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowSmall<64>>(const KArgs);
 
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_fwd_t<BF16, 128>(a, stream);

@@ -25,6 +25,7 @@ struct KArgs {
   int has_seq, causal, chunk;
   int nqt;   // query tiles per (batch, query head)
   float scale;
+  int compute_units;  // of the device the launch goes to (host-side launch-shape decisions)
 };
 
 }  // namespace moda

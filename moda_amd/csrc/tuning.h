@@ -1,13 +1,36 @@
-// Compile-time launch shapes of the streaming kernels.
+// Compile-time launch shapes of the streaming (query-row) kernels: forward and dQ.
 #pragma once
 
 namespace moda {
 
-// forward and dQ kernels: waves per workgroup (32 query rows each), LDS ring stages of
-// one 64-column K tile + V tile, and how many tiles ahead the global->LDS loads run.
-constexpr int kRowWaves = 8;
-constexpr int kRowStages = 3;
-constexpr int kRowDist = 2;
-constexpr int kRowBM = 32 * kRowWaves;  // query rows per workgroup
+// Waves per workgroup (32 query rows each), LDS ring stages of one 64-column K tile + V tile, and how
+// many tiles ahead the global->LDS loads run.
+//
+// RowLarge is the throughput shape: 256 query rows share every K/V tile.  RowSmall is for problems
+// with few query rows per (batch, head), where the large shape leaves compute units without a
+// workgroup and makes every wave sit through the barriers of depth tiles that only other waves of
+// its workgroup touch: fewer rows per workgroup mean more workgroups and a depth range that is
+// mostly the wave's own.  Its wave count is the smallest one whose tile loader covers a multiple
+// of 16 rows per pass (the LDS swizzle repeats every 16 rows).
+struct RowLarge {
+  static constexpr int W = 8, NST = 3, DIST = 2;
+};
+template <int HD>
+struct RowSmall;
+template <>
+struct RowSmall<64> {
+  static constexpr int W = 2, NST = 3, DIST = 2;  // 48 KB of LDS: three workgroups per compute unit
+};
+template <>
+struct RowSmall<128> {
+  static constexpr int W = 4, NST = 2, DIST = 1;  // 64 KB of LDS: two workgroups per compute unit
+};
+
+// Host side: the small shape is used when the large one would not even give every compute unit
+// two workgroups.
+inline bool use_small_rows(long long rows_per_head, long long heads, int compute_units) {
+  const long long large_blocks = (rows_per_head + 32 * RowLarge::W - 1) / (32 * RowLarge::W) * heads;
+  return large_blocks < 2ll * compute_units;
+}
 
 }  // namespace moda
