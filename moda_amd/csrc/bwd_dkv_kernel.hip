@@ -357,20 +357,111 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   }
 }
 
+// Depth columns outside chunk-visible mode (moda_v14.py:1251-1454, fda_v12.py:646-860): a depth slot is seen
+// by the G query rows of its own token only, so its gradients are 2*G dot products and 2*G scaled row
+// additions of length D -- far too little to fill a 64 x 128 MFMA tile, and on short sequences the
+// matrix kernel's per-workgroup latency dominated it.  Here HD/8 lanes share a column (16 bytes of the
+// head dim each), a wave covers 8 (D = 64) or 4 (D = 128) consecutive columns, everything stays in
+// registers and the kernel streams kd, vd in and dkd, dvd out once: it is bound by HBM.
+// P and dS are rounded to the input type before they are used, as in the matrix kernels.
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a) {
+  constexpr int LPC = HD / 8, CPW = 64 / LPC, CPB = 4 * CPW;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = lane % LPC;
+  const int BHk = a.B * a.Hkv;
+  const int bh = blockIdx.x % BHk;
+  const int b = bh / a.Hkv, hkv = bh % a.Hkv;
+  const int64_t c = (int64_t)(blockIdx.x / BHk) * CPB + wave * CPW + lane / LPC;
+  if (c >= (int64_t)a.T * a.L) return;  // whole lane groups leave together
+  const int w = (int)(c / a.L), slot = (int)(c - (int64_t)w * a.L);
+  uint16_t* dk_out = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + c * a.sdkd.t + 8 * sub;
+  uint16_t* dv_out = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + c * a.sdvd.t + 8 * sub;
+  if (slot >= a.Lv) {  // a slot without data
+    const i32x4 z = {0, 0, 0, 0};
+    *reinterpret_cast<i32x4*>(dk_out) = z;
+    *reinterpret_cast<i32x4*>(dv_out) = z;
+    return;
+  }
+  auto load8 = [&](const uint16_t* p, float (&f)[8]) {
+    const i32x4 v = *reinterpret_cast<const i32x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; i++) unpack2<T>(v[i], f[2 * i], f[2 * i + 1]);
+  };
+  float kf[8], vf[8], dk[8], dv[8];
+  load8(a.kd + b * a.skd.b + hkv * a.skd.h + c * a.skd.t + 8 * sub, kf);
+  load8(a.vd + b * a.svd.b + hkv * a.svd.h + c * a.svd.t + 8 * sub, vf);
+#pragma unroll
+  for (int i = 0; i < 8; i++) dk[i] = dv[i] = 0.f;
+  const float sc = a.scale * kLog2e;
+  const uint16_t* qb = a.q + b * a.sq.b + hkv * a.sq.h + 8 * sub;
+  const uint16_t* dob = a.d_o + b * a.sdo.b + hkv * a.sdo.h + 8 * sub;
+  for (int gq = 0; gq < a.Gf; gq++) {
+    const int64_t r = (int64_t)w * a.Gf + gq;
+    float qf[8], dof[8];
+    load8(qb + r * a.sq.t, qf);
+    load8(dob + r * a.sdo.t, dof);
+    float s = 0.f, dp = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      s = __builtin_fmaf(qf[i], kf[i], s);
+      dp = __builtin_fmaf(dof[i], vf[i], dp);
+    }
+#pragma unroll
+    for (int m = 1; m < LPC; m <<= 1) {
+      s += __shfl_xor(s, m, 64);
+      dp += __shfl_xor(dp, m, 64);
+    }
+    const float lse = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hkv];
+    const float neg_delta = a.delta[((int64_t)b * a.Hq + hkv) * a.Tq + r];
+    float p = fast_exp2(__builtin_fmaf(s, sc, -lse));
+    float ds = p * (dp + neg_delta);
+    unpack2<T>(pack2<T>(p, ds), p, ds);  // the rounding the matrix kernels apply before the second product
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      dv[i] = __builtin_fmaf(p, dof[i], dv[i]);
+      dk[i] = __builtin_fmaf(ds, qf[i], dk[i]);
+    }
+  }
+  i32x4 ok, ov;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    ok[i] = pack2<T>(dk[2 * i] * a.scale, dk[2 * i + 1] * a.scale);
+    ov[i] = pack2<T>(dv[2 * i], dv[2 * i + 1]);
+  }
+  *reinterpret_cast<i32x4*>(dk_out) = ok;
+  *reinterpret_cast<i32x4*>(dv_out) = ov;
+}
+
 template <typename T, int HD>
 hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = 3 * 2 * 64 * HD * sizeof(uint16_t) + 2 * 4 * 4 * 64 * 16 + 3 * 2 * 64 * sizeof(float);
   static LdsAttrState attr;
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_kernel<T, HD>), smem);
   if (ea != hipSuccess) return ea;
+  // depth columns: vector kernel, except in chunk-visible mode where a column has up to G*Cb visible rows
+  const bool depth_by_columns = a.L > 0 && !a.chunk;
   const int64_t n_seq_tiles = a.has_seq ? (a.T + 127) / 128 : 0;
-  const int64_t n_dep_tiles = a.L > 0 ? ((int64_t)a.T * a.L + 127) / 128 : 0;
+  const int64_t n_dep_tiles = (a.L > 0 && !depth_by_columns) ? ((int64_t)a.T * a.L + 127) / 128 : 0;
   const int64_t nblk = (n_seq_tiles + n_dep_tiles) * a.B * a.Hkv;
-  if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((dkv_kernel<T, HD>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
+  if (nblk > 0) {
+    hipLaunchKernelGGL((dkv_kernel<T, HD>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  if (depth_by_columns && (int64_t)a.B * a.T > 0) {
+    constexpr int CPB = 4 * (64 / (HD / 8));
+    const int64_t nx = (((int64_t)a.T * a.L + CPB - 1) / CPB) * a.B * a.Hkv;
+    if (nx >= (1ll << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((depth_cols_kernel<T, HD>), dim3((unsigned)nx), dim3(256), 0, stream, a);
+  }
   return hipGetLastError();
 }
 
+template __global__ void depth_cols_kernel<BF16, 128>(const KArgs);
+template __global__ void depth_cols_kernel<BF16, 64>(const KArgs);
+template __global__ void depth_cols_kernel<FP16, 128>(const KArgs);
+template __global__ void depth_cols_kernel<FP16, 64>(const KArgs);
 template __global__ void dkv_kernel<BF16, 128>(const KArgs);
 template __global__ void dkv_kernel<BF16, 64>(const KArgs);
 template __global__ void dkv_kernel<FP16, 128>(const KArgs);
