@@ -14,6 +14,7 @@
 // loop over column tiles is split in two: tiles every row of the workgroup sees
 // completely run a body without any masking or visibility tests; boundary and
 // depth tiles run the masked body.
+#include <algorithm>
 #include <type_traits>
 
 #include "kargs.h"
@@ -22,7 +23,7 @@
 
 namespace moda {
 
-template <typename T, int HD, typename Shape>
+template <typename T, int HD, typename Shape, bool WIDE>
 __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
   constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST,
                 DIST = Shape::DIST;
@@ -84,7 +85,12 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
     dep0 = lo_t * a.L;
     n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
   }
-  const int ntiles = n_seq + n_dep;
+  // wave-uniform by construction, but computed with vector divisions: the explicit hint keeps the
+  // loop control in scalar registers
+  n_seq = __builtin_amdgcn_readfirstlane(n_seq);
+  n_full = __builtin_amdgcn_readfirstlane(n_full);
+  dep0 = __builtin_amdgcn_readfirstlane(dep0);
+  const int ntiles = __builtin_amdgcn_readfirstlane(n_seq + n_dep);
 
   typedef AsyncTileLoader<HD, BN, NT> Loader;
   constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
@@ -105,8 +111,17 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
       srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
-    ld.load_from(Kt, srcK, row0);
-    ld.load_from(Kt + BN * HD, srcV, row0);
+    if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
+      const bool dep = it >= n_seq;
+      const int row_end = dep ? a.T * a.L : a.T;
+      ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
+              row0, row_end);
+      ld.load(Kt + BN * HD, dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h,
+              dep ? a.svd.t : a.sv.t, row0, row_end);
+    } else {
+      ld.load_from(Kt, srcK, row0);
+      ld.load_from(Kt + BN * HD, srcV, row0);
+    }
     ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
   };
   // wait until tile `next` has landed; tiles next+1 .. next+DIST-1 may still be in flight
@@ -235,32 +250,42 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
   }
 }
 
-template <typename T, int HD, typename Shape>
+template <typename T, int HD, typename Shape, bool WIDE>
 hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
   static LdsAttrState attr;
-  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD, Shape>), smem);
+  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD, Shape, WIDE>), smem);
   if (ea != hipSuccess) return ea;
   const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((fwd_kernel<T, HD, Shape>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
+  hipLaunchKernelGGL((fwd_kernel<T, HD, Shape, WIDE>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
   return hipGetLastError();
 }
 
 template <typename T, int HD>
 hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
-  if (use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units)) return launch_fwd_t_shape<T, HD, RowSmall<HD>>(a, stream);
-  return launch_fwd_t_shape<T, HD, RowLarge>(a, stream);
+  // byte span of the widest streamed (batch, head) slice
+  const int64_t span = 2 * std::max(std::max((int64_t)a.T * a.sk.t, (int64_t)a.T * a.sv.t),
+                                    std::max((int64_t)a.T * a.L * a.skd.t, (int64_t)a.T * a.L * a.svd.t));
+  const bool wide = span > 0x7fffffffll;
+  const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
+  if (wide) return launch_fwd_t_shape<T, HD, RowLarge, true>(a, stream);
+  if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, false>(a, stream);
+  return launch_fwd_t_shape<T, HD, RowLarge, false>(a, stream);
 }
 
-template __global__ void fwd_kernel<BF16, 128, RowLarge>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowLarge>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowLarge>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowLarge>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowSmall<128>>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowSmall<64>>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowSmall<128>>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowSmall<64>>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowLarge, false>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowLarge, false>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowLarge, false>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowLarge, false>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowLarge, true>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowLarge, true>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowLarge, true>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowLarge, true>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, false>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, false>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, false>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, false>(const KArgs);
 
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_fwd_t<BF16, 128>(a, stream);

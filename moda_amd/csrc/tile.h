@@ -397,11 +397,12 @@ struct AsyncTileLoader {
     row_in_pass = wave * RPW + lane / CH;
     gchunk = (lane % CH) ^ Tile<HD>::swz(row_in_pass);
   }
-  // A source of rows: fixed descriptor over rows [row_base, row_end) of a (batch, head) slice.
+  // A source of rows: fixed descriptor over rows [row_base, row_end) of a (batch, head) slice whose
+  // byte span fits 31 bits (kernels that may meet wider slices use load() below, which anchors a
+  // descriptor at every tile at the price of 64-bit address arithmetic per tile).
   struct Source {
     const uint16_t* base;  // row `row_base` of the slice
-    uint32_t nbytes;       // bytes from there to the end of the slice (used when they fit 31 bits)
-    int64_t total_bytes;   // the same, unclamped
+    uint32_t nbytes;       // bytes from there to the end of the slice
     int voff;              // this lane's byte offset inside a tile
     int stride_bytes;
     int row_base;
@@ -412,26 +413,14 @@ struct AsyncTileLoader {
     s.row_base = row_base;
     const int64_t nbytes = (int64_t)(row_end > row_base ? row_end - row_base : 0) * s.stride_bytes;
     s.base = slice + (int64_t)row_base * row_stride;
-    s.total_bytes = nbytes;
     s.nbytes = nbytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)nbytes;
     s.voff = row_in_pass * s.stride_bytes + gchunk * 16;
     return s;
   }
   // rows [row0, row0 + ROWS) of the source into `tile`; rows past the source's end arrive as zeros
   __device__ __forceinline__ void load_from(lds_ptr tile, const Source& s, int row0) const {
-    i32x4 rs;
-    int soff;
-    if (s.total_bytes > 0x7fffffffll) {
-      // the slice spans more than 32-bit offsets reach: anchor the descriptor at the tile itself
-      const int64_t off = (int64_t)(row0 - s.row_base) * s.stride_bytes;
-      const int64_t left = s.total_bytes - off;
-      rs = rsrc_words(reinterpret_cast<const char*>(s.base) + off,
-                      left <= 0 ? 0u : (uint32_t)(left > 0x7fffffffll ? 0x7fffffffll : left));
-      soff = 0;
-    } else {
-      rs = rsrc_words(s.base, s.nbytes);
-      soff = (row0 - s.row_base) * s.stride_bytes;
-    }
+    const int soff = (row0 - s.row_base) * s.stride_bytes;
+    const i32x4 rs = rsrc_words(s.base, s.nbytes);
 #pragma unroll
     for (int i = 0; i < N; i++)
       lds_dma<16>(rs, lds_addr(tile + (i * NW + wave) * 512), s.voff, soff + i * NW * RPW * s.stride_bytes);
