@@ -288,13 +288,17 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
       for (int k = 0; k < kParts; k++) part(k);
       end_trip();
     };
-    auto body = [&](auto masked_tag, int rel_qt) {
+    // `stage_tag`: the ring stage as a compile-time constant (the tile's LDS offset then rides in the
+    // immediate field of every operand read) or -1 = take it from c_st
+    auto body = [&](auto masked_tag, auto stage_tag, int rel_qt) {
       constexpr bool MASKED = decltype(masked_tag)::value;
+      constexpr int STAGE = decltype(stage_tag)::value;
       const int q0 = (qt0 + rel_qt) * BM;
-      lds_cptr Qs = ring + c_st * 2 * BM * HD;
+      const int st = STAGE >= 0 ? STAGE : c_st;
+      lds_cptr Qs = ring + st * 2 * BM * HD;
       lds_cptr dOs = Qs + BM * HD;
       MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * 4 * 64 + lane;
-      MODA_LDS const float* st_s = stat + c_st * 2 * BM;
+      MODA_LDS const float* st_s = stat + st * 2 * BM;
       bool run = true;
       if (MASKED) {
         run = __any((qhi > q0) && (qlo < q0 + BM) && (qhi > qlo));
@@ -312,17 +316,27 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
       c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
       c_par ^= 1;
     };
+    using dyn = std::integral_constant<int, -1>;
     if (ROLE_B) idle_trip();
     for (int gh = 0; gh < a.hdiv; gh++) {
       int rel_qt = nqt - 1;
-      for (; rel_qt >= first_free_qt; rel_qt--) {
+      auto free_trip = [&](auto stage_tag) {
         begin_trip();
-        body(std::false_type{}, rel_qt);
+        body(std::false_type{}, stage_tag, rel_qt);
         end_trip();
+        rel_qt--;
+      };
+      // unmasked tiles: reach ring stage 0, then three trips per round with the stage known at compile time
+      while (rel_qt >= first_free_qt && c_st != 0) free_trip(dyn{});
+      while (rel_qt - (NST - 1) >= first_free_qt) {
+        free_trip(std::integral_constant<int, 0>{});
+        free_trip(std::integral_constant<int, 1>{});
+        free_trip(std::integral_constant<int, 2>{});
       }
+      while (rel_qt >= first_free_qt) free_trip(dyn{});
       for (; rel_qt >= 0; rel_qt--) {
         begin_trip();
-        body(std::true_type{}, rel_qt);
+        body(std::true_type{}, dyn{}, rel_qt);
         end_trip();
       }
     }

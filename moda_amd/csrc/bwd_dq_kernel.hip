@@ -193,8 +193,11 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a) {
     kt.run(oa, Kc, DS, dq);
   };
 
-  // phase 1: tiles fully visible to every row -- no masks, no visibility tests
-  for (int it = 0; it < n_full; it++) {
+  // phase 1: tiles fully visible to every row -- no masks, no visibility tests.  (Not unrolled over the
+  // ring stages like the forward loop: this kernel has no registers left for a second set of operand
+  // addresses.)
+  int it = 0;
+  for (; it < n_full; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     lds_cptr Kc = smem + c_st * 2 * BN * HD;
     tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, 0, 0);
@@ -203,7 +206,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a) {
     __syncthreads();
   }
   // phase 2: boundary sequence tiles and depth tiles
-  for (int it = n_full; it < ntiles; it++) {
+  for (; it < ntiles; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     const bool dep = it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;

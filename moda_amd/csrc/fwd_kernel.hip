@@ -208,17 +208,30 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
     pv.run(oa, Vc, P, o);
   };
 
-  // phase 1: tiles fully visible to every row -- no masks, no visibility tests
-  for (int it = 0; it < n_full; it++) {
+  // phase 1: tiles fully visible to every row -- no masks, no visibility tests.  The loop is unrolled
+  // over the ring stages so that each copy reads its tile at a compile-time LDS offset (the stage
+  // offset then rides in the instructions' immediate field instead of costing an address add per
+  // operand read); the remainder runs the same body with the stage in a register.
+  int it = 0;
+  auto full_tile = [&](lds_cptr Kc) {
     if (it + DIST < ntiles) issue(it + DIST);
-    lds_cptr Kc = smem + c_st * 2 * BN * HD;
     tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, 0, 0);
-    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
     wait_tile(it + 1);
     __syncthreads();
+    it++;
+  };
+  for (; it + NST <= n_full;) {
+    full_tile(smem);
+    full_tile(smem + 1 * 2 * BN * HD);
+    if (NST > 2) full_tile(smem + 2 * 2 * BN * HD);
+  }
+  c_st = 0;
+  for (; it < n_full;) {
+    full_tile(smem + c_st * 2 * BN * HD);
+    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
   }
   // phase 2: boundary sequence tiles and depth tiles
-  for (int it = n_full; it < ntiles; it++) {
+  for (; it < ntiles; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     const bool dep = it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
