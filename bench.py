@@ -30,7 +30,10 @@ WORKLOADS = {
     "c5": (64, 197, 6, 1, 64, 12, "noncausal", 0),
     "c5fda": (64, 197, 6, 1, 64, 12, "depth_only", 0),
     "plain": (1, 65536, 4, 4, 128, 0, "plain", 0),
+    # the c4 token count as one packed variable-length batch (cu_seqlens): 1 x 16K, 2 x 8K, 4 x 4K, 8 x 2K tokens
+    "c4packed": (1, 65536, 4, 4, 128, 24, "causal", 0),
 }
+PACKED_LENGTHS = {"c4packed": [16384] + [8192] * 2 + [4096] * 4 + [2048] * 8}
 
 
 def flops_fwd(B, T, Hq, D, L, mode, cb):
@@ -239,13 +242,20 @@ def main():
                    "depth_only": _lib.DEPTH_ONLY}[mode]
             Garg = G
         state = {}
+        packed = None
+        if name in PACKED_LENGTHS:
+            cu = [0]
+            for n_tok in PACKED_LENGTHS[name]:
+                cu.append(cu[-1] + n_tok)
+            assert cu[-1] == T
+            packed = ops._packed(torch.tensor(cu, dtype=torch.int32, device=dev), q, G)
 
         def fwd():
-            state["o"], state["lse"] = ops._raw_fwd(mid, q, k, v, kd, vd, sc, Garg, cb)
+            state["o"], state["lse"] = ops._raw_fwd(mid, q, k, v, kd, vd, sc, Garg, cb, packed=packed)
 
         def bwd(stages=_lib.STAGE_ALL):
             state["grads"] = ops._raw_bwd(mid, q, k, v, kd, vd, state["o"], state["lse"], do, sc, Garg, cb,
-                                          stages=stages, out=state.get("grads"), ws=state.get("ws"))
+                                          stages=stages, out=state.get("grads"), ws=state.get("ws"), packed=packed)
 
         fwd()
         state["ws"] = torch.empty(B * Hkv * G * T * 4 + 16, dtype=torch.uint8, device=dev)
@@ -277,7 +287,10 @@ def main():
         t_dq = ev_time(lambda: bwd(_lib.STAGE_DQ), n)
         t_dkv = ev_time(lambda: bwd(_lib.STAGE_DKV), n)
         Hq = Hkv * G
-        ff = flops_fwd(B, T, Hq, D, L, mode, cb)
+        if packed is not None:
+            ff = sum(flops_fwd(1, n_tok, Hq, D, L, mode, cb) for n_tok in PACKED_LENGTHS[name])
+        else:
+            ff = flops_fwd(B, T, Hq, D, L, mode, cb)
         return {"ms_step": ms_step, "flops_fwd": ff, "t_fwd": t_fwd, "t_delta": t_delta, "t_dq": t_dq,
                 "t_dkv": t_dkv, "shape": (B, T, Hkv, G, D, L, mode, cb)}
 
@@ -345,7 +358,9 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {mode} B={B} T={T} Hq={Hkv * G} Hkv={Hkv} G={G} D={D} L={L}"
-                               + (f" chunk_tokens={cb}" if cb else ""),
+                               + (f" chunk_tokens={cb}" if cb else "")
+                               + (f" packed sequence lengths={PACKED_LENGTHS[args.workload]}"
+                                  if args.workload in PACKED_LENGTHS else ""),
                    "flop_fwd_bwd": total_flops},
         "frac_of_bf16_mfma_peak": value / PEAK_BF16_TFLOPS,
         "kernels": kernels,

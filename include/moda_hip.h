@@ -29,6 +29,18 @@
  * [B, T*L_valid, H, D], and dkd, dvd are written as zeros in the other slots.
  * The invisible slots are still read (and multiplied by zero): they must hold
  * finite values.  Not available with MODA_HIP_CHUNK_VISIBLE.
+ *
+ * Packed variable-length batch (the reference carries a cu_seqlens argument but asserts
+ * it away, moda_v14.py:83-101, 2672-2673): with cu_seqlens != NULL the tensors have no
+ * batch axis (batch strides are ignored); sequence i of the B sequences owns base tokens
+ * [cu_seqlens[i], cu_seqlens[i+1]) of one packed token axis of total_tokens tokens, i.e.
+ * query rows cu*G .., key rows cu .., depth rows cu*L .. of q [total*G, H, D],
+ * k [total, H, D], kd [total*L, H, D], lse [total*G, H].  Offsets count BASE TOKENS
+ * (equal to query rows when G == 1), start at 0 and do not decrease; T is the length of
+ * the longest sequence.  Sequences attend only within themselves; chunks of
+ * CHUNK_VISIBLE are counted from each sequence's first token.  The offsets are read on
+ * the device only: the host cannot check them, rows outside [0, total_tokens) named by
+ * them are out-of-bounds accesses.
  */
 #ifndef MODA_HIP_H_
 #define MODA_HIP_H_
@@ -40,7 +52,7 @@
 extern "C" {
 #endif
 
-#define MODA_HIP_VERSION 101
+#define MODA_HIP_VERSION 102
 
 enum moda_hip_dtype { MODA_HIP_BF16 = 0, MODA_HIP_FP16 = 1, MODA_HIP_FP32 = 2 };
 
@@ -83,6 +95,8 @@ typedef struct moda_hip_desc {
   float scale;          /* logits = scale * <q, key>                               */
   float reserved_f;
   moda_hip_strides q, k, v, kd, vd, o, d_o, dq, dk, dv, dkd, dvd;
+  const int32_t* cu_seqlens; /* packed variable-length batch (see above): DEVICE array of B + 1 offsets, else NULL */
+  int64_t total_tokens;      /* with cu_seqlens: cu_seqlens[B], the length of the packed token axis              */
 } moda_hip_desc;
 
 /*

@@ -61,6 +61,8 @@ class Desc(Structure):
         ("dv", Strides),
         ("dkd", Strides),
         ("dvd", Strides),
+        ("cu_seqlens", c_void_p),
+        ("total_tokens", c_int64),
     ]
 
 

@@ -40,8 +40,8 @@ __device__ __forceinline__ void unpack2<FP16>(int w, float& lo, float& hi) {
   hi = (float)v[1];
 }
 
-template <typename T, int HD>
-__global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
+template <typename T, int HD, bool VARLEN>
+__global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   constexpr int BN = 128, BM = 64, KK = HD / 16, DB = HD / 32, NST = 3;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
@@ -54,14 +54,19 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kblk = wave & 3;
   const bool role_b = wave >= 4;
-  const int BHk = a.B * a.Hkv;
+  const int BHk = a_in.B * a_in.Hkv;
   const int bh = blockIdx.x % BHk;
   const int ct = blockIdx.x / BHk;
-  const int b = bh / a.Hkv, hkv = bh % a.Hkv;
-  const int n_seq_tiles = a.has_seq ? (a.T + BN - 1) / BN : 0;
+  int b = bh / a_in.Hkv;
+  const int hkv = bh % a_in.Hkv;
+  // the grid holds the sequence tiles of the longest sequence, then (when launched with them) the depth tiles
+  const int n_seq_tiles = a_in.has_seq ? (a_in.T + BN - 1) / BN : 0;
+  SeqArgs<VARLEN> seq(a_in, b);
+  const KArgs& a = seq.a;
   const bool dep = ct >= n_seq_tiles;
   const int ncols = dep ? a.T * a.L : a.T;
   const int c_first = (dep ? ct - n_seq_tiles : ct) * BN;
+  if (VARLEN && c_first >= ncols) return;  // a tile beyond this sequence of a variable-length batch
   const int c = c_first + kblk * 32 + n;
   const bool valid = c < ncols;
   // a depth slot without data: no row sees it; its K/V are replaced by zeros, its gradients come out zero
@@ -135,7 +140,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
     q_ptr = (const char*)(a.q + b * a.sq.b + hq * a.sq.h + (int64_t)f_q0 * a.sq.t);
     do_ptr = (const char*)(a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)f_q0 * a.sdo.t);
     st_ptr = wave == 0 ? (const char*)(a.lse + ((int64_t)b * a.Tq + f_q0) * a.Hq + hq)
-                       : (const char*)(a.delta + ((int64_t)b * a.Hq + hq) * a.Tq + f_q0);
+                       : (const char*)(a.delta + ((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + f_q0);
     ld_gh++;
   };
   i32x4 rs_q, rs_do, rs_stat;
@@ -379,13 +384,16 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a) {
 // registers and the kernel streams kd, vd in and dkd, dvd out once: it is bound by HBM.
 // P and dS are rounded to the input type before they are used, as in the matrix kernels.
 template <typename T, int HD>
-__global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a) {
+__global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   constexpr int LPC = HD / 8, CPW = 64 / LPC, CPB = 4 * CPW;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int sub = lane % LPC;
+  KArgs a = a_in;
   const int BHk = a.B * a.Hkv;
   const int bh = blockIdx.x % BHk;
-  const int b = bh / a.Hkv, hkv = bh % a.Hkv;
+  int b = bh / a.Hkv;
+  const int hkv = bh % a.Hkv;
+  enter_sequence(a, b);
   const int64_t c = (int64_t)(blockIdx.x / BHk) * CPB + wave * CPW + lane / LPC;
   if (c >= (int64_t)a.T * a.L) return;  // whole lane groups leave together
   const int w = (int)(c / a.L), slot = (int)(c - (int64_t)w * a.L);
@@ -427,7 +435,7 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a) {
       dp += __shfl_xor(dp, m, 64);
     }
     const float lse = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hkv];
-    const float neg_delta = a.delta[((int64_t)b * a.Hq + hkv) * a.Tq + r];
+    const float neg_delta = a.delta[((int64_t)b * a.Hq + hkv) * a.delta_pitch + r];
     float p = fast_exp2(__builtin_fmaf(s, sc, -lse));
     float ds = p * (dp + neg_delta);
     unpack2<T>(pack2<T>(p, ds), p, ds);  // the rounding the matrix kernels apply before the second product
@@ -451,7 +459,10 @@ template <typename T, int HD>
 hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = 3 * 2 * 64 * HD * sizeof(uint16_t) + 2 * 4 * 4 * 64 * 16 + 3 * 2 * 64 * sizeof(float);
   static LdsAttrState attr;
-  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_kernel<T, HD>), smem);
+  static LdsAttrState attr_packed;
+  const hipError_t ea =
+      a.cu ? allow_dynamic_lds(attr_packed, reinterpret_cast<const void*>(&dkv_kernel<T, HD, true>), smem)
+           : allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_kernel<T, HD, false>), smem);
   if (ea != hipSuccess) return ea;
   // depth columns: vector kernel, except in chunk-visible mode where a column has up to G*Cb visible rows
   const bool depth_by_columns = a.L > 0 && !a.chunk;
@@ -459,7 +470,10 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   const int64_t n_dep_tiles = (a.L > 0 && !depth_by_columns) ? ((int64_t)a.T * a.L + 127) / 128 : 0;
   const int64_t nblk = (n_seq_tiles + n_dep_tiles) * a.B * a.Hkv;
   if (nblk > 0) {
-    hipLaunchKernelGGL((dkv_kernel<T, HD>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
+    if (a.cu)
+      hipLaunchKernelGGL((dkv_kernel<T, HD, true>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
+    else
+      hipLaunchKernelGGL((dkv_kernel<T, HD, false>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -476,10 +490,14 @@ template __global__ void depth_cols_kernel<BF16, 128>(const KArgs);
 template __global__ void depth_cols_kernel<BF16, 64>(const KArgs);
 template __global__ void depth_cols_kernel<FP16, 128>(const KArgs);
 template __global__ void depth_cols_kernel<FP16, 64>(const KArgs);
-template __global__ void dkv_kernel<BF16, 128>(const KArgs);
-template __global__ void dkv_kernel<BF16, 64>(const KArgs);
-template __global__ void dkv_kernel<FP16, 128>(const KArgs);
-template __global__ void dkv_kernel<FP16, 64>(const KArgs);
+template __global__ void dkv_kernel<BF16, 128, false>(const KArgs);
+template __global__ void dkv_kernel<BF16, 128, true>(const KArgs);
+template __global__ void dkv_kernel<BF16, 64, false>(const KArgs);
+template __global__ void dkv_kernel<BF16, 64, true>(const KArgs);
+template __global__ void dkv_kernel<FP16, 128, false>(const KArgs);
+template __global__ void dkv_kernel<FP16, 128, true>(const KArgs);
+template __global__ void dkv_kernel<FP16, 64, false>(const KArgs);
+template __global__ void dkv_kernel<FP16, 64, true>(const KArgs);
 
 hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_dkv_t<BF16, 128>(a, stream);

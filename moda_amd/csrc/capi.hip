@@ -74,6 +74,15 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   a.chunk = d->mode == MODA_HIP_CHUNK_VISIBLE;
   a.nqt = (a.Tq + 127) / 128;
   a.scale = d->scale;
+  a.delta_pitch = a.Tq;
+  if (d->cu_seqlens) {
+    // packed batch: T is the longest sequence, the row axes hold total_tokens tokens
+    if (d->total_tokens < d->T || ((uintptr_t)d->cu_seqlens % 4) != 0) return MODA_HIP_EINVAL;
+    if (d->total_tokens * d->G >= (1ll << 30) || d->total_tokens * (d->L > 0 ? d->L : 1) >= (1ll << 30))
+      return MODA_HIP_EUNSUPPORTED;
+    a.cu = d->cu_seqlens;
+    a.delta_pitch = (int)(plain ? d->total_tokens : d->total_tokens * d->G);
+  }
   return MODA_HIP_OK;
 }
 
@@ -156,7 +165,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
 size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* d) {
   KArgs a;
   if (fill_geometry(d, a)) return 0;
-  const size_t n = (size_t)a.B * a.Hq * a.Tq * sizeof(float);
+  const size_t n = (a.cu ? (size_t)1 : (size_t)a.B) * a.Hq * a.delta_pitch * sizeof(float);
   return n ? n : sizeof(float);
 }
 

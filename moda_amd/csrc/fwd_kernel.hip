@@ -23,8 +23,10 @@
 
 namespace moda {
 
-template <typename T, int HD, typename Shape, bool WIDE>
-__global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
+// ADDR: 0 = 32-bit offsets inside a (batch, head) slice; 1 = slices wider than 2 GiB (descriptors anchored
+// per tile); 2 = packed variable-length batch (per-tile descriptors as well)
+template <typename T, int HD, typename Shape, int ADDR>
+__global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in) {
   constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST,
                 DIST = Shape::DIST;
   static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
@@ -32,11 +34,16 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
   lds_ptr smem = (lds_ptr)smem_raw;  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
-  const int BH = a.B * a.Hq;
+  constexpr bool WIDE = ADDR != 0, VARLEN = ADDR == 2;
+  const int BH = a_in.B * a_in.Hq;
   const int bh = blockIdx.x % BH;
+  int b = bh / a_in.Hq;
+  const int hq = bh % a_in.Hq, hkv = hq / a_in.hdiv;
+  SeqArgs<VARLEN> seq(a_in, b);
+  const KArgs& a = seq.a;
   const int nqt = (a.Tq + BM - 1) / BM;
   const int qt = nqt - 1 - blockIdx.x / BH;  // heavy (late) tiles first
-  const int b = bh / a.Hq, hq = bh % a.Hq, hkv = hq / a.hdiv;
+  if (VARLEN && qt < 0) return;                        // a tile beyond this sequence of a variable-length batch
   const int r = qt * BM + wave * 32 + n;
   const bool valid = r < a.Tq;
   const int t = r / a.Gf;
@@ -263,15 +270,15 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a) {
   }
 }
 
-template <typename T, int HD, typename Shape, bool WIDE>
+template <typename T, int HD, typename Shape, int ADDR>
 hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
   static LdsAttrState attr;
-  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD, Shape, WIDE>), smem);
+  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;
   const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
-  hipLaunchKernelGGL((fwd_kernel<T, HD, Shape, WIDE>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
+  hipLaunchKernelGGL((fwd_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
   return hipGetLastError();
 }
 
@@ -282,23 +289,35 @@ hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
                                     std::max((int64_t)a.T * a.L * a.skd.t, (int64_t)a.T * a.L * a.svd.t));
   const bool wide = span > 0x7fffffffll;
   const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
-  if (wide) return launch_fwd_t_shape<T, HD, RowLarge, true>(a, stream);
-  if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, false>(a, stream);
-  return launch_fwd_t_shape<T, HD, RowLarge, false>(a, stream);
+  if (a.cu) {
+    if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, 2>(a, stream);
+    return launch_fwd_t_shape<T, HD, RowLarge, 2>(a, stream);
+  }
+  if (wide) return launch_fwd_t_shape<T, HD, RowLarge, 1>(a, stream);
+  if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, 0>(a, stream);
+  return launch_fwd_t_shape<T, HD, RowLarge, 0>(a, stream);
 }
 
-template __global__ void fwd_kernel<BF16, 128, RowLarge, false>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowLarge, false>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowLarge, false>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowLarge, false>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowLarge, true>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowLarge, true>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowLarge, true>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowLarge, true>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, false>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, false>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, false>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, false>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, 0>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, 0>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, 0>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, 0>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, 2>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, 2>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, 2>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, 2>(const KArgs);
 
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_fwd_t<BF16, 128>(a, stream);

@@ -37,13 +37,17 @@ struct RowGeom {
   int shi, dlo, dhi;
 };
 
-__device__ __forceinline__ bool row_geom(const KArgs& a, int64_t gid, RowGeom& g) {
+// `a` arrives as launched and leaves rebased on the row's sequence (variable-length batches)
+template <typename E>
+__device__ __forceinline__ bool row_geom(KArgs& a, int64_t gid, RowGeom& g) {
   const int64_t total = (int64_t)a.B * a.Hq * a.Tq;
   if (gid >= total) return false;
   g.r = (int)(gid % a.Tq);
   const int bh = (int)(gid / a.Tq);
   g.b = bh / a.Hq;
   g.hq = bh % a.Hq;
+  enter_sequence(a, g.b, sizeof(E) / 2);
+  if (g.r >= a.Tq) return false;  // a row beyond this sequence
   g.hkv = g.hq / a.hdiv;
   g.t = g.r / a.Gf;
   g.shi = a.has_seq ? (a.causal ? g.t + 1 : a.T) : 0;
@@ -58,13 +62,14 @@ __device__ __forceinline__ bool row_geom(const KArgs& a, int64_t gid, RowGeom& g
 
 // MODE 0: forward (o, lse).  MODE 1: dq (needs lse; delta computed inline).
 template <typename E, int MODE>
-__global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a, const int D) {
+__global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, const int D) {
   __shared__ float qs[4][kMaxD];
   __shared__ float dos[4][kMaxD];
   __shared__ float pb[4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   RowGeom g;
-  if (!row_geom(a, (int64_t)blockIdx.x * 4 + wave, g)) return;  // whole wave exits together
+  KArgs a = a_in;
+  if (!row_geom<E>(a, (int64_t)blockIdx.x * 4 + wave, g)) return;  // whole wave exits together
   const int64_t qoff = g.b * a.sq.b + g.hq * a.sq.h + (int64_t)g.r * a.sq.t;
   const int64_t dooff = g.b * a.sdo.b + g.hq * a.sdo.h + (int64_t)g.r * a.sdo.t;
   const int64_t ooff = g.b * a.so.b + g.hq * a.so.h + (int64_t)g.r * a.so.t;
@@ -163,21 +168,25 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a, const i
 
 // dK/dV: one wave per column (sequence key or depth slot) of one (batch, kv head).
 template <typename E>
-__global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a, const int D) {
+__global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, const int D) {
   __shared__ float kc[4][kMaxD];
   __shared__ float vc[4][kMaxD];
   __shared__ float pb[4][64];
   __shared__ float dsb[4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  KArgs a = a_in;
   const int n_seq = a.has_seq ? a.T : 0;
   const int ncol = n_seq + a.T * a.L;
   const int64_t gid = (int64_t)blockIdx.x * 4 + wave;
   if (gid >= (int64_t)a.B * a.Hkv * ncol) return;
   const int cidx = (int)(gid % ncol);
   const int bh = (int)(gid / ncol);
-  const int b = bh / a.Hkv, hkv = bh % a.Hkv;
+  int b = bh / a.Hkv;
+  const int hkv = bh % a.Hkv;
+  enter_sequence(a, b, sizeof(E) / 2);
   const bool dep = cidx >= n_seq;
   const int col = dep ? cidx - n_seq : cidx;
+  if (col >= (dep ? a.T * a.L : a.T)) return;  // a column beyond this sequence
   const void* kp = dep ? (const void*)a.kd : (const void*)a.k;
   const void* vp = dep ? (const void*)a.vd : (const void*)a.v;
   const Str3 ks = dep ? a.skd : a.sk, vs = dep ? a.svd : a.sv;

@@ -1,5 +1,6 @@
 // Kernel argument block shared by the host launchers and the device kernels.
 #pragma once
+#include <hip/hip_runtime.h>
 #include <stdint.h>
 
 namespace moda {
@@ -12,7 +13,7 @@ struct KArgs {
   const uint16_t *q, *k, *v, *kd, *vd, *o, *d_o;
   uint16_t *out_o, *dq, *dk, *dv, *dkd, *dvd;
   float* lse;          // [B, Tq, Hq]   (written by forward, read by backward)
-  float* delta;        // [B, Hq, Tq]   workspace: MINUS rowsum(o * do)
+  float* delta;        // [B, Hq, delta_pitch]   workspace: MINUS rowsum(o * do)
   Str3 sq, sk, sv, skd, svd, so, sdo, sdq, sdk, sdv, sdkd, sdvd;
   int B, T, Hkv;
   int Tq;    // query rows per (batch, query head)
@@ -26,6 +27,54 @@ struct KArgs {
   int nqt;   // query tiles per (batch, query head)
   float scale;
   int compute_units;  // of the device the launch goes to (host-side launch-shape decisions)
+  // Packed variable-length batch: cu[b] .. cu[b+1] are the base tokens of sequence b on a row axis all
+  // sequences share (the tensors have no batch axis then); T, Tq above are those of the longest sequence.
+  const int32_t* cu;
+  int delta_pitch;  // query rows per head in `delta`: Tq, or the packed total
+};
+
+// Variable-length batches: rebases every tensor on the first row of sequence `b` and shrinks T / Tq to the
+// sequence's length, so that the code after it addresses the sequence as batch 0 of a fixed-length problem.
+// The launch grid is sized for the longest sequence: callers drop the tiles beyond their own sequence.
+// `units`: 16-bit units per tensor element (the data pointers are typed for 16-bit elements).
+__device__ __forceinline__ void enter_sequence(KArgs& a, int& b, int units = 1) {
+  if (a.cu == nullptr) return;
+  const int t0 = a.cu[b];
+  const int T = a.cu[b + 1] - t0;
+  const int64_t r0 = (int64_t)t0 * a.Gf * units, c0 = (int64_t)t0 * a.L * units, k0 = (int64_t)t0 * units;
+  a.q += r0 * a.sq.t;
+  a.o += r0 * a.so.t;
+  a.d_o += r0 * a.sdo.t;
+  a.out_o += r0 * a.so.t;
+  a.dq += r0 * a.sdq.t;
+  a.k += k0 * a.sk.t;
+  a.v += k0 * a.sv.t;
+  a.dk += k0 * a.sdk.t;
+  a.dv += k0 * a.sdv.t;
+  a.kd += c0 * a.skd.t;
+  a.vd += c0 * a.svd.t;
+  a.dkd += c0 * a.sdkd.t;
+  a.dvd += c0 * a.sdvd.t;
+  a.lse += (int64_t)t0 * a.Gf * a.Hq;
+  a.delta += (int64_t)t0 * a.Gf;
+  a.T = T;
+  a.Tq = T * a.Gf;
+  b = 0;
+}
+
+// The argument block a kernel body works on: the launch's own (fixed-length instantiations, no copy)
+// or a copy rebased on the workgroup's sequence.
+template <bool VARLEN>
+struct SeqArgs;
+template <>
+struct SeqArgs<false> {
+  const KArgs& a;
+  __device__ __forceinline__ SeqArgs(const KArgs& in, int&) : a(in) {}
+};
+template <>
+struct SeqArgs<true> {
+  KArgs a;
+  __device__ __forceinline__ SeqArgs(const KArgs& in, int& b) : a(in) { enter_sequence(a, b); }
 };
 
 }  // namespace moda

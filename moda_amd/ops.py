@@ -18,7 +18,7 @@ from __future__ import annotations
 
 import ctypes
 import warnings
-from typing import Optional, Tuple
+from typing import NamedTuple, Optional, Tuple
 
 import torch
 
@@ -30,6 +30,37 @@ _DTYPES = {torch.bfloat16: _lib.BF16, torch.float16: _lib.FP16, torch.float32: _
 # Query rows per chunk of the chunk-visible variant when the caller does not
 # say: the value the reference hard-wires in its launchers (moda_v16.py:581-585).
 DEFAULT_CHUNK_ROWS = 64
+
+
+class PackedBatch(NamedTuple):
+    """A variable-length batch on one packed token axis, as the kernels take it."""
+    cu: torch.Tensor  # int32 [n + 1] on the device: first base token of each sequence, then the total
+    n: int            # sequences
+    max_len: int      # base tokens of the longest sequence
+    total: int        # base tokens in the packed axis
+
+
+def _packed(cu_seqlens, q: torch.Tensor, rows_per_token: int) -> Optional[PackedBatch]:
+    """``cu_seqlens`` as a caller passes it (fla's convention: cumulative sequence lengths, first entry 0,
+    tensors of batch size 1 holding all sequences back to back) -> PackedBatch.  The offsets count BASE
+    TOKENS, i.e. rows of k/v; sequence i owns query rows ``cu[i]*G .. cu[i+1]*G`` and depth rows
+    ``cu[i]*L .. cu[i+1]*L``.  The reference carries the argument but asserts it away
+    (moda_v14.py:2672-2673); its dormant kernel code reads the offsets in query rows (moda_v14.py:83-101),
+    which is the same thing for ``moda_group_num == 1``.  Costs one device-to-host copy of the offsets
+    (the longest sequence sizes the launch); pass the returned PackedBatch instead of the tensor to reuse it."""
+    if cu_seqlens is None or isinstance(cu_seqlens, PackedBatch):
+        return cu_seqlens
+    assert q.shape[0] == 1, "with cu_seqlens all sequences share one packed row axis: batch size must be 1"
+    assert cu_seqlens.dim() == 1 and cu_seqlens.numel() >= 1, "cu_seqlens must be a vector of n+1 offsets"
+    host = cu_seqlens.detach().to("cpu", torch.int64)
+    lens = host[1:] - host[:-1]
+    assert int(host[0]) == 0 and bool((lens >= 0).all()), "cu_seqlens must start at 0 and not decrease"
+    total = int(host[-1])
+    assert total * rows_per_token == q.shape[1], (
+        f"cu_seqlens ends at {total} base tokens but q holds {q.shape[1]} rows "
+        f"({rows_per_token} per token)")
+    cu = cu_seqlens.detach().to(device=q.device, dtype=torch.int32).contiguous()
+    return PackedBatch(cu, int(lens.numel()), int(lens.max()) if lens.numel() else 0, total)
 
 
 def _ptr(x: Optional[torch.Tensor]):
@@ -72,7 +103,7 @@ def _check_device(x: torch.Tensor):
 
 
 def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=None, dk=None, dv=None, dkd=None,
-          dvd=None, depth_valid=None) -> Desc:
+          dvd=None, depth_valid=None, packed: Optional[PackedBatch] = None) -> Desc:
     d = Desc()
     d.struct_size = ctypes.sizeof(Desc)
     if q.dtype not in _DTYPES:
@@ -92,6 +123,10 @@ def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=
         d.T = q.shape[1] // G
     else:
         d.T = k.shape[1]
+    if packed is not None:
+        d.B, d.T = packed.n, packed.max_len
+        d.cu_seqlens = packed.cu.data_ptr()
+        d.total_tokens = packed.total
     d.chunk_tokens = chunk_tokens
     d.scale = float(scale)
     d.q, d.k, d.v, d.kd, d.vd = _strides(q), _strides(k), _strides(v), _strides(kd), _strides(vd)
@@ -111,7 +146,7 @@ def _same_dtype(*xs):
             raise TypeError(f"all tensors must share one dtype, got {dt} and {x.dtype}")
 
 
-def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None):
+def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None, packed=None):
     """Launch the forward kernels. Returns (o, lse)."""
     _check_device(q)
     _same_dtype(q, k, v, kd, vd)
@@ -128,7 +163,7 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None):
     lse = torch.empty(q.shape[0], q.shape[1], q.shape[2], dtype=torch.float32, device=q.device)
     if L == 0:
         kd = vd = None
-    d = _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=o, depth_valid=depth_valid)
+    d = _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=o, depth_valid=depth_valid, packed=packed)
     with torch.cuda.device(q.device):
         rc = _lib.load().moda_hip_fwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kd), _ptr(vd), _ptr(o),
                                       _ptr(lse), _stream(q))
@@ -137,7 +172,7 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None):
 
 
 def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages=_lib.STAGE_ALL, out=None, ws=None,
-             depth_valid=None):
+             depth_valid=None, packed=None):
     """Launch the backward kernels. Returns (dq, dk, dv, dkd, dvd).
 
     ``stages`` selects a subset of {delta, dq, dk/dv}; ``out`` (a previous return
@@ -158,7 +193,7 @@ def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages
         dvd = torch.empty(vd.shape, dtype=vd.dtype, device=q.device) if vd is not None else None
     kd_a, vd_a, dkd_a, dvd_a = (kd, vd, dkd, dvd) if L > 0 else (None, None, None, None)
     d = _desc(mode, q, k, v, kd_a, vd_a, G, L, chunk_tokens, scale, o=o, do=do, dq=dq, dk=dk, dv=dv, dkd=dkd_a,
-              dvd=dvd_a, depth_valid=depth_valid)
+              dvd=dvd_a, depth_valid=depth_valid, packed=packed)
     lib = _lib.load()
     nbytes = lib.moda_hip_bwd_workspace_bytes(ctypes.byref(d))
     if ws is None:
@@ -188,7 +223,6 @@ def parallel_moda_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, 
     ``depth_valid`` (not in the reference): only the first ``depth_valid`` of the ``L`` slots per token
     of ``cached_k/v`` are visible."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
-    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
     assert q.shape[2] == k.shape[2], (
         "Implicit head-dimension GQA is not allowed. "
         "Please fold grouping only into `moda_group_num`: "
@@ -196,7 +230,8 @@ def parallel_moda_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, 
     )
     _assert_group_tile(moda_group_num)
     mode = _lib.CAUSAL if is_causal else _lib.NONCAUSAL
-    return _raw_fwd(mode, q, k, v, cached_k, cached_v, scale, moda_group_num, depth_valid=depth_valid)
+    return _raw_fwd(mode, q, k, v, cached_k, cached_v, scale, moda_group_num, depth_valid=depth_valid,
+                    packed=_packed(cu_seqlens, q, moda_group_num))
 
 
 def parallel_moda_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None, cached_k=None,
@@ -205,7 +240,6 @@ def parallel_moda_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128,
                       group_warps=None, depth_bs=None, depth_warps=None, depth_valid=None):
     """moda_v14.py:1470-1842.  Returns ``(dq, dk, dv, dg_cumsum=None, d_cached_k, d_cached_v)``."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
-    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
     assert q.shape[2] == k.shape[2], (
         "Implicit head-dimension GQA is not allowed. "
         "Please fold grouping only into `moda_group_num`: "
@@ -216,18 +250,19 @@ def parallel_moda_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128,
     _assert_group_tile(moda_group_num)
     mode = _lib.CAUSAL if is_causal else _lib.NONCAUSAL
     dq, dk, dv, dkd, dvd = _raw_bwd(mode, q, k, v, cached_k, cached_v, o, lse, do, scale, moda_group_num,
-                                    depth_valid=depth_valid)
+                                    depth_valid=depth_valid, packed=_packed(cu_seqlens, q, moda_group_num))
     return dq, dk, dv, None, dkd, dvd
 
 
 def _autograd_forward(ctx, fwd_impl, q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, **kw):
     assert g is None, "g is not supported in this version"
-    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
+    packed = _packed(cu_seqlens, q, moda_group_num)
     has_depth = cached_k is not None and cached_v is not None
     if not has_depth:
         cached_k = cached_v = None
-    o, lse = fwd_impl(q=q, k=k, v=v, g_cumsum=None, scale=scale, cu_seqlens=None, cached_k=cached_k,
+    o, lse = fwd_impl(q=q, k=k, v=v, g_cumsum=None, scale=scale, cu_seqlens=packed, cached_k=cached_k,
                       cached_v=cached_v, moda_group_num=moda_group_num, **kw)
+    ctx.packed = packed
     ctx.save_for_backward(q, k, v, o, lse, *([cached_k, cached_v] if has_depth else []))
     ctx.has_depth = has_depth
     ctx.scale = scale
@@ -243,7 +278,7 @@ def _autograd_backward(ctx, bwd_impl, do):
         q, k, v, o, lse = ctx.saved_tensors
         cached_k = cached_v = None
     dq, dk, dv, _, dkd, dvd = bwd_impl(q=q, k=k, v=v, o=o, g_cumsum=None, lse=lse, do=do.to(o.dtype), scale=ctx.scale,
-                                       cu_seqlens=None, cached_k=cached_k, cached_v=cached_v,
+                                       cu_seqlens=ctx.packed, cached_k=cached_k, cached_v=cached_v,
                                        moda_group_num=ctx.moda_group_num, **ctx.kw)
     if not ctx.has_depth:
         dkd = dvd = None
@@ -357,10 +392,10 @@ def parallel_moda_chunk_visible_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, c
                                     customized_BV=None, customized_num_warps=None):
     """moda_v16.py:498-633.  ``customized_BT`` is the chunk size in query rows (default 64)."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
-    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
     assert q.shape[2] == k.shape[2], "Implicit head-dimension GQA is not allowed."
     cb = _chunk_tokens(moda_group_num, customized_BT)
-    return _raw_fwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, scale, moda_group_num, cb)
+    return _raw_fwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, scale, moda_group_num, cb,
+                    packed=_packed(cu_seqlens, q, moda_group_num))
 
 
 def parallel_moda_chunk_visible_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None,
@@ -369,12 +404,11 @@ def parallel_moda_chunk_visible_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, c
                                     customized_num_warps=None):
     """moda_v16.py:2099-2343."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
-    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
     if scale is None:
         scale = q.shape[-1] ** -0.5
     cb = _chunk_tokens(moda_group_num, customized_BT)
     dq, dk, dv, dkd, dvd = _raw_bwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, o, lse, do, scale,
-                                    moda_group_num, cb)
+                                    moda_group_num, cb, packed=_packed(cu_seqlens, q, moda_group_num))
     return dq, dk, dv, None, dkd, dvd
 
 
@@ -421,10 +455,10 @@ def parallel_fda_fwd(q, g_cumsum, scale, cu_seqlens=None, cached_k=None, cached_
                      customized_num_warps=None):
     """fda_v12.py:261-400.  Returns ``(o, lse)``."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
-    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
     assert cached_k is not None and cached_v is not None, "Flash Depth Attention requires cached_k/cached_v"
     _assert_group_tile(moda_group_num)
-    return _raw_fwd(_lib.DEPTH_ONLY, q, None, None, cached_k, cached_v, scale, moda_group_num)
+    return _raw_fwd(_lib.DEPTH_ONLY, q, None, None, cached_k, cached_v, scale, moda_group_num,
+                    packed=_packed(cu_seqlens, q, moda_group_num))
 
 
 def parallel_fda_bwd(q, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None, cached_k=None,
@@ -433,11 +467,10 @@ def parallel_fda_bwd(q, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seq
                      depth_warps=None):
     """fda_v12.py:881-1135.  Returns ``(dq, dg_cumsum=None, d_cached_k, d_cached_v)``."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
-    assert cu_seqlens is None, "cu_seqlens is not supported in this version"
     if scale is None:
         scale = q.shape[-1] ** -0.5
     dq, _, _, dkd, dvd = _raw_bwd(_lib.DEPTH_ONLY, q, None, None, cached_k, cached_v, o, lse, do, scale,
-                                  moda_group_num)
+                                  moda_group_num, packed=_packed(cu_seqlens, q, moda_group_num))
     return dq, None, dkd, dvd
 
 
@@ -449,9 +482,9 @@ class ParallelFlashDepthAttentionFunction(torch.autograd.Function):
     def forward(ctx, q, k, v, g, scale, cu_seqlens, cached_k=None, cached_v=None, moda_group_num=1, group_bs=None,
                 group_warps=None, depth_bs=None, depth_warps=None):
         assert g is None, "g is not supported in this version"
-        assert cu_seqlens is None, "cu_seqlens is not supported in this version"
         assert k is None and v is None, "Flash Depth Attention does not accept legacy k/v; pass None"
-        o, lse = parallel_fda_fwd(q, None, scale, None, cached_k, cached_v, moda_group_num)
+        ctx.packed = _packed(cu_seqlens, q, moda_group_num)
+        o, lse = parallel_fda_fwd(q, None, scale, ctx.packed, cached_k, cached_v, moda_group_num)
         ctx.save_for_backward(q, o, lse, cached_k, cached_v)
         ctx.scale = scale
         ctx.moda_group_num = moda_group_num
@@ -462,8 +495,8 @@ class ParallelFlashDepthAttentionFunction(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, do, dlse_unused):
         q, o, lse, cached_k, cached_v = ctx.saved_tensors
-        dq, _, dkd, dvd = parallel_fda_bwd(q, o, None, lse, do.to(o.dtype), ctx.scale, cached_k=cached_k,
-                                           cached_v=cached_v, moda_group_num=ctx.moda_group_num)
+        dq, _, dkd, dvd = parallel_fda_bwd(q, o, None, lse, do.to(o.dtype), ctx.scale, cu_seqlens=ctx.packed,
+                                           cached_k=cached_k, cached_v=cached_v, moda_group_num=ctx.moda_group_num)
         return dq.to(q), None, None, None, None, None, dkd, dvd, None, None, None, None, None
 
 
@@ -521,20 +554,22 @@ def parallel_fda(q, k=None, v=None, g=None, cached_k=None, cached_v=None, scale=
 # ---------------------------------------------------------------------------
 def parallel_attn_fwd(q, k, v, g_cumsum=None, scale=None, cu_seqlens=None):
     """fla/ops/attn/parallel.py:443-503.  q ``[B,T,HQ,D]``, k/v ``[B,T,H,D]``; returns ``(o, lse)``."""
-    assert g_cumsum is None and cu_seqlens is None
+    assert g_cumsum is None
     assert q.shape[2] % k.shape[2] == 0, "HQ must be a multiple of H"
     assert q.shape[1] == k.shape[1]
     if scale is None:
         scale = k.shape[-1] ** -0.5
-    return _raw_fwd(_lib.PLAIN_GQA, q, k, v, None, None, scale, q.shape[2] // k.shape[2])
+    return _raw_fwd(_lib.PLAIN_GQA, q, k, v, None, None, scale, q.shape[2] // k.shape[2],
+                    packed=_packed(cu_seqlens, q, 1))
 
 
 def parallel_attn_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None):
     """fla/ops/attn/parallel.py:522-629.  Returns ``(dq, dk, dv, dg=None)``."""
-    assert g_cumsum is None and cu_seqlens is None
+    assert g_cumsum is None
     if scale is None:
         scale = k.shape[-1] ** -0.5
-    dq, dk, dv, _, _ = _raw_bwd(_lib.PLAIN_GQA, q, k, v, None, None, o, lse, do, scale, q.shape[2] // k.shape[2])
+    dq, dk, dv, _, _ = _raw_bwd(_lib.PLAIN_GQA, q, k, v, None, None, o, lse, do, scale, q.shape[2] // k.shape[2],
+                                packed=_packed(cu_seqlens, q, 1))
     return dq, dk, dv, None
 
 
@@ -545,8 +580,8 @@ class ParallelAttentionFunction(torch.autograd.Function):
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, q, k, v, g, scale, cu_seqlens):
         assert g is None, "g is not supported"
-        assert cu_seqlens is None, "cu_seqlens is not supported"
-        o, lse = parallel_attn_fwd(q, k, v, None, scale, None)
+        ctx.packed = _packed(cu_seqlens, q, 1)
+        o, lse = parallel_attn_fwd(q, k, v, None, scale, ctx.packed)
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.scale = scale
         return o.to(q.dtype)
@@ -555,7 +590,7 @@ class ParallelAttentionFunction(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, do):
         q, k, v, o, lse = ctx.saved_tensors
-        dq, dk, dv, _ = parallel_attn_bwd(q, k, v, o, None, lse, do.to(o.dtype), ctx.scale)
+        dq, dk, dv, _ = parallel_attn_bwd(q, k, v, o, None, lse, do.to(o.dtype), ctx.scale, cu_seqlens=ctx.packed)
         return dq.to(q), dk.to(k), dv.to(v), None, None, None
 
 

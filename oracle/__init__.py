@@ -17,6 +17,8 @@ from .moda_oracle import (  # noqa: F401
     depth_cache_grad_ref,
     compact_depth,
     scatter_depth_grad,
+    packed_visible_mask,
+    moda_packed_fwd_bwd,
     make_inputs,
     error_metrics,
     passes_reference_rule,

@@ -259,6 +259,74 @@ def scatter_depth_grad(g: torch.Tensor, T: int, L: int) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------
+# packed variable-length batches (an extension of this build; the reference carries a cu_seqlens
+# argument but asserts it away, moda_v14.py:2672-2673)
+# --------------------------------------------------------------------------
+def packed_visible_mask(cu: Sequence[int], G: int, L: int, mode: str, chunk_tokens: int = 0) -> torch.Tensor:
+    """Boolean mask ``[total*G, total + total*L]`` of a packed batch, written out element by element.
+
+    ``cu`` are cumulative sequence lengths in base tokens.  A query row sees a column iff both belong to
+    the same sequence and the rule of :func:`visible_mask` holds for their positions counted from the
+    sequence's first token (so chunks of the chunk-visible variant restart with every sequence)."""
+    total = int(cu[-1])
+    seq_of, local = [], []
+    for i in range(len(cu) - 1):
+        for t in range(int(cu[i]), int(cu[i + 1])):
+            seq_of.append(i)
+            local.append(t - int(cu[i]))
+    m = torch.zeros(total * G, total + total * L, dtype=torch.bool)
+    for r in range(total * G):
+        t = r // G
+        for j in range(total):
+            if seq_of[j] != seq_of[t]:
+                continue
+            if mode in ("causal", "chunk_visible"):
+                m[r, j] = local[j] <= local[t]
+            elif mode == "noncausal":
+                m[r, j] = True
+        for c in range(total * L):
+            w = c // L
+            if seq_of[w] != seq_of[t]:
+                continue
+            if mode == "chunk_visible":
+                start = (local[t] // chunk_tokens) * chunk_tokens
+                m[r, total + c] = start <= local[w] <= local[t]
+            else:
+                m[r, total + c] = w == t
+    return m
+
+
+def moda_packed_fwd_bwd(inp: Dict[str, torch.Tensor], cu: Sequence[int], scale, G, mode, chunk_tokens=0,
+                        dtype=torch.float32):
+    """:func:`moda_dense_fwd_bwd` for a packed batch: tensors of batch size 1 hold the sequences back to
+    back (sequence i = base tokens ``cu[i] .. cu[i+1]``, query rows ``cu*G``, depth rows ``cu*L``); every
+    sequence is evaluated on its own and the results are put back in place.  This DEFINES the
+    ``cu_seqlens`` option of the kernels."""
+    total = int(cu[-1])
+    L = inp["kd"].shape[1] // total if (inp.get("kd") is not None and total > 0) else 0
+    span = {"q": G, "do": G, "k": 1, "v": 1, "kd": L, "vd": L}
+    res = {}
+    for name in ("o", "dq"):
+        res[name] = torch.zeros(inp["q"].shape, dtype=dtype)
+    res["lse"] = torch.zeros(inp["q"].shape[:3], dtype=dtype)
+    for name in ("k", "v", "kd", "vd"):
+        res["d" + name] = None if inp.get(name) is None else torch.zeros(inp[name].shape, dtype=dtype)
+    for i in range(len(cu) - 1):
+        a, b = int(cu[i]), int(cu[i + 1])
+        if a == b:
+            continue
+        part = {n: (None if inp.get(n) is None else inp[n][:, a * m:b * m]) for n, m in span.items()}
+        r = moda_dense_fwd_bwd(part, scale, G, mode, chunk_tokens, dtype)
+        res["o"][:, a * G:b * G] = r["o"]
+        res["lse"][:, a * G:b * G] = r["lse"]
+        res["dq"][:, a * G:b * G] = r["dq"]
+        for n in ("k", "v", "kd", "vd"):
+            if r["d" + n] is not None:
+                res["d" + n][:, a * span[n]:b * span[n]] = r["d" + n]
+    return res
+
+
+# --------------------------------------------------------------------------
 # (iii) blockwise evaluation with explicit gradient formulas
 # --------------------------------------------------------------------------
 @torch.no_grad()

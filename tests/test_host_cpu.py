@@ -32,8 +32,9 @@ def test_descriptor_layout_and_version():
     from moda_amd import _lib
 
     lib = _lib.load()
-    assert lib.moda_hip_version() == 101
-    assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24
+    assert lib.moda_hip_version() == 102
+    assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24 + 16
+    assert _lib.Desc.cu_seqlens.offset == 80 + 12 * 24
     assert _lib.Desc.q.offset == 80
     # a descriptor with the wrong struct_size is rejected without touching any device
     d = _lib.Desc()
@@ -61,6 +62,12 @@ def test_descriptor_validation_codes():
     assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc())) == 8 * 4
     assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc(G=4, H=2, B=3))) == 3 * 2 * 32 * 4
     assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc(mode=_lib.PLAIN_GQA, G=4, H=2))) == 8 * 8 * 4
+    # packed variable-length batch: the workspace covers the packed row axis once, not B x longest sequence
+    assert lib.moda_hip_bwd_workspace_bytes(
+        ctypes.byref(desc(B=3, T=8, G=2, H=2, cu_seqlens=0x1000, total_tokens=13))) == 2 * 13 * 2 * 4
+    # ... the longest sequence cannot exceed the packed axis; the offsets must be 4-byte aligned
+    assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc(B=3, T=8, cu_seqlens=0x1000, total_tokens=7))) == 0
+    assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(desc(B=3, T=8, cu_seqlens=0x1002, total_tokens=9))) == 0
     null = None
     # missing q pointer
     assert lib.moda_hip_fwd(ctypes.byref(desc()), null, null, null, null, null, null, null, null) == -1
@@ -118,11 +125,19 @@ def test_argument_contract_matches_reference():
     with pytest.raises(AssertionError, match="head count"):
         moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), cached_k=z(1, 16, 1, 64),
                                cached_v=z(1, 16, 1, 64))
-    # g / cu_seqlens are unsupported (moda_v14.py:2672-2673)
+    # g is unsupported (moda_v14.py:2672); cu_seqlens, which the reference asserts away in the next line,
+    # is accepted here and validated on the host
     with pytest.raises(AssertionError, match="g is not supported"):
         moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), g=torch.zeros(1, 8, 2))
-    with pytest.raises(AssertionError, match="cu_seqlens is not supported"):
-        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), cu_seqlens=torch.tensor([0, 8]))
+    with pytest.raises(AssertionError, match="batch size must be 1"):
+        moda_amd.parallel_moda(z(2, 8, 2, 64), z(2, 8, 2, 64), z(2, 8, 2, 64), cu_seqlens=torch.tensor([0, 8]))
+    with pytest.raises(AssertionError, match="start at 0 and not decrease"):
+        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), cu_seqlens=torch.tensor([0, 5, 3, 8]))
+    with pytest.raises(AssertionError, match="ends at 7 base tokens"):
+        moda_amd.parallel_moda(z(1, 16, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), moda_group_num=2,
+                               cu_seqlens=torch.tensor([0, 3, 7]))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        moda_amd.parallel_moda(z(1, 8, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), cu_seqlens=torch.tensor([0, 3, 8]))
     # group size must divide the query tile (moda_v14.py:476-478)
     with pytest.raises(AssertionError, match="BT % moda_group_num"):
         moda_amd.parallel_moda(z(1, 24, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64), moda_group_num=3)

@@ -281,3 +281,42 @@ def test_compact_and_scatter_depth_are_adjoint_slot_selections():
     for t in range(T):
         for l in range(valid, L):
             assert x.grad[:, t * L + l].abs().max() == 0
+
+
+@pytest.mark.parametrize("mode,G,L,cb", [("causal", 1, 2, 0), ("causal", 2, 3, 0), ("noncausal", 2, 1, 0),
+                                          ("chunk_visible", 2, 2, 2), ("depth_only", 2, 3, 0), ("causal", 1, 0, 0)])
+def test_packed_batch_is_block_masked_attention_over_the_packed_axis(mode, G, L, cb):
+    """The per-sequence evaluation that defines cu_seqlens equals ONE library softmax over the whole packed
+    axis under a mask written out element by element (same sequence AND the variant's rule on positions
+    counted from the sequence start), forward and all gradients: pins which rows belong to which
+    sequence (q rows cu*G, depth rows cu*L)."""
+    cu = [0, 3, 3, 4, 9]  # lengths 3, 0, 1, 5
+    total, H, D = cu[-1], 2, 8
+    g = torch.Generator().manual_seed(11)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    inp = {"q": r(1, total * G, H, D), "do": r(1, total * G, H, D)}
+    if mode != "depth_only":
+        inp["k"], inp["v"] = r(1, total, H, D), r(1, total, H, D)
+    if L:
+        inp["kd"], inp["vd"] = r(1, total * L, H, D), r(1, total * L, H, D)
+    scale = 0.3
+    got = oracle.moda_packed_fwd_bwd(inp, cu, scale, G, mode, cb, dtype=torch.float64)
+
+    mask = oracle.packed_visible_mask(cu, G, L, mode, cb)
+    leaf = {n: x.clone().requires_grad_(True) for n, x in inp.items() if n != "do"}
+    keys = [leaf["k"] if "k" in leaf else torch.zeros(1, total, H, D, dtype=torch.float64)]
+    vals = [leaf["v"] if "v" in leaf else torch.zeros(1, total, H, D, dtype=torch.float64)]
+    if L:
+        keys.append(leaf["kd"])
+        vals.append(leaf["vd"])
+    kc, vc = torch.cat(keys, 1).transpose(1, 2), torch.cat(vals, 1).transpose(1, 2)
+    o = F.scaled_dot_product_attention(leaf["q"].transpose(1, 2), kc, vc, attn_mask=mask.view(1, 1, *mask.shape),
+                                       scale=scale).transpose(1, 2)
+    (o * inp["do"]).sum().backward()
+    assert torch.allclose(got["o"], o.detach(), atol=1e-12)
+    for n in ("q", "k", "v", "kd", "vd"):
+        if n in leaf:
+            assert torch.allclose(got["d" + n], leaf[n].grad, atol=1e-11), n
+    logits = torch.einsum("bqhd,bhkd->bhqk", inp["q"], kc.detach()) * scale
+    lse = torch.logsumexp(logits.masked_fill(~mask, float("-inf")), -1).permute(0, 2, 1) / math.log(2.0)
+    assert torch.allclose(got["lse"], lse, atol=1e-12)

@@ -589,6 +589,97 @@ def test_mfma_probe_runs(gpu_device):
     assert lib.moda_hip_mfma_probe(None, 1, 1, None, ctypes.c_void_p(sink.data_ptr()), None) == -1  # MODA_HIP_EINVAL
 
 
+# ---------------------------------------------------------------------------
+# packed variable-length batches (cu_seqlens): the oracle evaluates every sequence on its own
+# ---------------------------------------------------------------------------
+PACKED = [
+    # lengths (base tokens), H, D, L, G, mode, chunk_tokens, dtype
+    ((300, 1, 0, 129, 64, 700), 2, 128, 3, 4, "causal", 0, torch.bfloat16),
+    ((197, 197, 50), 3, 64, 12, 1, "noncausal", 0, torch.bfloat16),
+    ((5, 260, 33), 2, 64, 2, 2, "noncausal", 0, torch.float16),
+    ((130, 17, 400), 1, 128, 6, 4, "chunk_visible", 16, torch.bfloat16),
+    ((64, 0, 65, 3), 2, 64, 5, 2, "chunk_visible", 32, torch.float16),
+    ((100, 7, 260), 2, 128, 7, 2, "depth_only", 0, torch.bfloat16),
+    ((1100,), 1, 128, 2, 1, "causal", 0, torch.bfloat16),
+    ((3, 2, 1, 1, 40), 2, 64, 0, 2, "causal", 0, torch.bfloat16),
+    ((70, 9, 31), 2, 32, 3, 2, "causal", 0, torch.float32),
+    ((40, 55), 1, 96, 2, 1, "noncausal", 0, torch.bfloat16),
+]
+
+
+def _cu(lengths):
+    cu = [0]
+    for n in lengths:
+        cu.append(cu[-1] + n)
+    return cu
+
+
+@pytest.mark.parametrize("case", PACKED, ids=lambda c: f"{c[5]}-{'_'.join(map(str, c[0]))}-D{c[2]}-L{c[3]}-G{c[4]}")
+def test_packed_variable_length_batches(gpu_device, case):
+    from moda_amd import ops
+
+    lengths, H, D, L, G, mode, cb, dtype = case
+    say(f"[packed] {case}")
+    cu = _cu(lengths)
+    total = cu[-1]
+    inp = oracle.make_inputs(1, total, H, D, L, G, seed=29, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
+    sc = D ** -0.5
+    ref = oracle.moda_packed_fwd_bwd(inp, cu, sc, G, mode, cb)
+    dev = to_dev(inp, gpu_device)
+    packed = ops._packed(torch.tensor(cu, device=gpu_device), dev["q"], G)
+    assert (packed.n, packed.max_len, packed.total) == (len(lengths), max(lengths), total)
+    m = MODE_ID[mode]
+    o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], sc, G, cb, packed=packed)
+    dq, dk, dv, dkd, dvd = ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], o, lse, dev["do"], sc, G,
+                                        cb, packed=packed)
+    got = {"o": o, "lse": lse, "dq": dq, "dk": dk, "dv": dv, "dkd": dkd, "dvd": dvd}
+    compare_all(got, ref, dtype, str(case))
+
+
+def test_packed_batch_equals_separate_calls_bitwise(gpu_device):
+    """One launch over the packed batch returns, bit for bit, what one call per sequence returns; also
+    through the public autograd interface with an int64 cu_seqlens as callers of fla pass it."""
+    import moda_amd
+
+    lengths, H, D, L, G = (333, 64, 1, 520), 2, 128, 4, 4
+    cu = _cu(lengths)
+    inp = to_dev(oracle.make_inputs(1, cu[-1], H, D, L, G, seed=31, dtype=torch.bfloat16, std=0.5), gpu_device)
+    leaf = {n: inp[n].clone().requires_grad_(True) for n in ("q", "k", "v", "kd", "vd")}
+    o, lse = moda_amd.parallel_moda(leaf["q"], leaf["k"], leaf["v"], cached_k=leaf["kd"], cached_v=leaf["vd"],
+                                    moda_group_num=G, need_lse=True,
+                                    cu_seqlens=torch.tensor(cu, dtype=torch.int64, device=gpu_device))
+    (o * inp["do"]).sum().backward()
+    mult = {"q": G, "k": 1, "v": 1, "kd": L, "vd": L}
+    for i in range(len(lengths)):
+        a, b = cu[i], cu[i + 1]
+        part = {n: inp[n][:, a * m:b * m] for n, m in mult.items()}
+        part["do"] = inp["do"][:, a * G:b * G]
+        one = run_hip(part, D ** -0.5, G, "causal")
+        assert torch.equal(o[:, a * G:b * G], one["o"]) and torch.equal(lse[:, a * G:b * G], one["lse"]), i
+        for n, key in (("q", "dq"), ("k", "dk"), ("v", "dv"), ("kd", "dkd"), ("vd", "dvd")):
+            assert torch.equal(leaf[n].grad[:, a * mult[n]:b * mult[n]], one[key]), (i, n)
+
+
+def test_packed_plain_gqa_attention(gpu_device):
+    import moda_amd
+
+    lengths, Hkv, G, D = (200, 77, 300), 2, 4, 128
+    cu = _cu(lengths)
+    inp = oracle.make_inputs(1, cu[-1], Hkv, D, 0, G, seed=37, dtype=torch.bfloat16, std=0.5, Hq=Hkv * G)
+    dev = to_dev(inp, gpu_device)
+    dl = {n: dev[n].clone().requires_grad_(True) for n in ("q", "k", "v")}
+    o = moda_amd.parallel_attn(dl["q"], dl["k"], dl["v"], cu_seqlens=torch.tensor(cu, device=gpu_device))
+    (o * dev["do"]).sum().backward()
+    for i in range(len(lengths)):
+        a, b = cu[i], cu[i + 1]
+        leaf = {n: inp[n][:, a:b].float().clone().requires_grad_(True) for n in ("q", "k", "v")}
+        o_ref, _ = oracle.plain_gqa_dense(leaf["q"], leaf["k"], leaf["v"])
+        (o_ref * inp["do"][:, a:b].float()).sum().backward()
+        check("o", o[:, a:b], o_ref, torch.bfloat16, f"packed plain {i}")
+        for n in ("q", "k", "v"):
+            check("d" + n, dl[n].grad[:, a:b], leaf[n].grad, torch.bfloat16, f"packed plain {i}")
+
+
 def test_empty_and_degenerate(gpu_device):
     import moda_amd
 
