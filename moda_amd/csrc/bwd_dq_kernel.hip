@@ -42,8 +42,8 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a_in) {
   if (r < a.Tq && (tid % TPR) == 0) a.delta[((int64_t)b * a.Hq + hq) * a.delta_pitch + r] = -acc;
 }
 
-// ADDR: 0 = 32-bit offsets inside a (batch, head) slice; 1 = slices wider than 2 GiB (descriptors anchored
-// per tile); 2 = packed variable-length batch (per-tile descriptors as well)
+// ADDR bit 0: a (batch, head) slice is wider than 2 GiB (descriptors anchored per tile instead of 32-bit
+// offsets inside the slice); bit 1: packed variable-length batch
 template <typename T, int HD, typename Shape, int ADDR>
 __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) {
   constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST, DIST = Shape::DIST;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
-  constexpr bool WIDE = ADDR != 0, VARLEN = ADDR == 2;
+  constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0;
   const int BH = a_in.B * a_in.Hq;
   const int bh = blockIdx.x % BH;
   int b = bh / a_in.Hq;
@@ -274,6 +274,7 @@ hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
   const bool wide = span > 0x7fffffffll;
   const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
   if (a.cu) {
+    if (wide) return launch_dq_t_shape<T, HD, RowLarge, 3>(a, stream);
     if (small) return launch_dq_t_shape<T, HD, RowSmall<HD>, 2>(a, stream);
     return launch_dq_t_shape<T, HD, RowLarge, 2>(a, stream);
   }
@@ -295,12 +296,16 @@ template __global__ void dq_kernel<BF16, 64, RowSmall<64>, 0>(const KArgs);
 template __global__ void dq_kernel<FP16, 128, RowSmall<128>, 0>(const KArgs);
 template __global__ void dq_kernel<FP16, 64, RowSmall<64>, 0>(const KArgs);
 template __global__ void dq_kernel<BF16, 128, RowLarge, 2>(const KArgs);
+template __global__ void dq_kernel<BF16, 128, RowLarge, 3>(const KArgs);
 template __global__ void dq_kernel<BF16, 128, RowSmall<128>, 2>(const KArgs);
 template __global__ void dq_kernel<BF16, 64, RowLarge, 2>(const KArgs);
+template __global__ void dq_kernel<BF16, 64, RowLarge, 3>(const KArgs);
 template __global__ void dq_kernel<BF16, 64, RowSmall<64>, 2>(const KArgs);
 template __global__ void dq_kernel<FP16, 128, RowLarge, 2>(const KArgs);
+template __global__ void dq_kernel<FP16, 128, RowLarge, 3>(const KArgs);
 template __global__ void dq_kernel<FP16, 128, RowSmall<128>, 2>(const KArgs);
 template __global__ void dq_kernel<FP16, 64, RowLarge, 2>(const KArgs);
+template __global__ void dq_kernel<FP16, 64, RowLarge, 3>(const KArgs);
 template __global__ void dq_kernel<FP16, 64, RowSmall<64>, 2>(const KArgs);
 
 hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream) {

@@ -457,6 +457,19 @@ def test_slices_wider_than_32bit_offsets(gpu_device):
     ref = oracle.moda_rows_subset(cpu, rows, D ** -0.5, G, "causal")
     check("o", b["o"][:, rows.to(gpu_device)], ref["o"], torch.bfloat16, "wide-slices")
     check("dq", b["dq"][:, rows.to(gpu_device)], ref["dq"], torch.bfloat16, "wide-slices")
+    # the same views as a packed variable-length batch
+    from moda_amd import ops
+
+    say("CASE wide-slices packed")
+    packed = ops._packed(torch.tensor([0, 1000, 1001, T], device=gpu_device), inp["q"], G)
+
+    def run_packed(x):
+        o, lse = ops._raw_fwd(0, x["q"], x["k"], x["v"], x["kd"], x["vd"], D ** -0.5, G, packed=packed)
+        return (o, lse) + tuple(ops._raw_bwd(0, x["q"], x["k"], x["v"], x["kd"], x["vd"], o, lse, x["do"], D ** -0.5, G,
+                                             packed=packed))
+
+    for i, (x, y) in enumerate(zip(run_packed(inp), run_packed(wide))):
+        assert torch.equal(x, y), i
 
 
 @pytest.mark.parametrize("case", [
