@@ -208,6 +208,44 @@ def bench_mfma_probe(dev):
     return out
 
 
+def bench_stack(dev, steps=10):
+    """Whole-model step around the operator: the twelve blocks of the reference's smallest MoDA vision
+    model (vision_tasks/deit/models.py:425-428: width 256, 4 query heads, 1 kv head, 197 tokens) at batch 64,
+    bf16 weights, chained through one depth stream.  Reported: training step (forward + backward, cache rebuilt
+    by the HIP reorganisation kernel), inference forward with the in-place cache, inference forward
+    rebuilding the cache per layer as the reference does."""
+    import torch
+
+    import moda_amd
+
+    torch.manual_seed(0)
+    dim, depth, heads, kv_heads, B, N = 256, 12, 4, 1, 64, 197
+    model = moda_amd.MoDAStack(dim, depth, heads, kv_heads).to(dev).to(torch.bfloat16)
+    x = (0.5 * torch.randn(B, N, dim, device=dev)).to(torch.bfloat16)
+
+    def train():
+        model.zero_grad(set_to_none=True)
+        model(x.clone().requires_grad_(True)).float().square().mean().backward()
+
+    def infer(inplace):
+        with torch.no_grad():
+            model(x, inplace_cache=inplace)
+
+    def timed(fn):
+        fn()
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    return {"config": f"12 blocks, width {dim}, {heads} heads / {kv_heads} kv head, B={B}, N={N}, bf16, noncausal",
+            "train_step_ms": timed(train), "inference_inplace_cache_ms": timed(lambda: infer(True)),
+            "inference_rebuilt_cache_ms": timed(lambda: infer(False))}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,6 +254,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--with-twin", action="store_true", help="also time the plain causal twin (c4 shape, no depth)")
+    ap.add_argument("--with-stack", action="store_true",
+                    help="also time a 12-block attention+MLP stack chained through the depth stream")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards over batch and kv heads without exchange "
@@ -376,6 +416,8 @@ def main():
     probe = bench_mfma_probe(dev)
     out["mfma_probe"] = probe
     out["frac_of_measured_mfma_rate"] = value / probe["random"]["tflops"]
+    if args.with_stack:
+        out["attention_stack"] = bench_stack(dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, T, Hkv, G, D, L, mode, cb)
     print(json.dumps(out))

@@ -23,6 +23,7 @@ from .ops import (  # noqa: F401
     ParallelAttentionFunction,
 )
 from .depth_cache import build_depth_cache, stack_depth, DepthCache  # noqa: F401
+from .modules import DepthStream, MoDAAttention, MoDAStack  # noqa: F401
 
 __all__ = [
     "parallel_moda",
@@ -40,4 +41,7 @@ __all__ = [
     "build_depth_cache",
     "stack_depth",
     "DepthCache",
+    "DepthStream",
+    "MoDAAttention",
+    "MoDAStack",
 ]

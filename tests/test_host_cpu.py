@@ -166,3 +166,21 @@ def test_compat_package_reexports():
         sys.path.pop(0)
         for m in [m for m in sys.modules if m == "fla" or m.startswith("fla.")]:
             del sys.modules[m]
+
+
+def test_attention_module_mirrors_reference_parameters():
+    """Parameter names and shapes of vision_tasks/deit/models.py:224-243 (a reference state_dict loads
+    unchanged); an empty depth stream yields no cache."""
+    import moda_amd
+
+    m = moda_amd.MoDAAttention(384, num_heads=6, num_kv_heads=3, qkv_bias=True)
+    shapes = {n: tuple(p.shape) for n, p in m.state_dict().items()}
+    assert shapes == {"q.weight": (384, 384), "q.bias": (384,), "kv.weight": (384, 384), "kv.bias": (384,),
+                      "proj.weight": (384, 384), "proj.bias": (384,)}
+    assert m.moda_group_num == 2 and m.head_dim == 64 and m.scale == 64 ** -0.5
+    with pytest.raises(ValueError, match="divisible by num_kv_heads"):
+        moda_amd.MoDAAttention(384, num_heads=6, num_kv_heads=4)
+    s = moda_amd.DepthStream(4)
+    assert s.context() == (None, None, None) and len(s) == 0
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        m(torch.zeros(1, 8, 384))

@@ -693,6 +693,58 @@ def test_packed_plain_gqa_attention(gpu_device):
             check("d" + n, dl[n].grad[:, a:b], leaf[n].grad, torch.bfloat16, f"packed plain {i}")
 
 
+# ---------------------------------------------------------------------------
+# the attention module and the depth-stream manager around the operator
+# ---------------------------------------------------------------------------
+def _oracle_parallel_moda(q, k, v, g=None, scale=None, cu_seqlens=None, cached_k=None, cached_v=None, moda_group_num=1,
+                          is_causal=True, head_first=False, warn_shape=True, depth_valid=None):
+    """What the module calls, answered by the oracle's dense form in fp32 and rounded to the input type."""
+    assert depth_valid is None
+    o, _ = oracle.moda_dense(q, k, v, cached_k, cached_v, scale, moda_group_num, "causal" if is_causal else "noncausal")
+    return o.to(q.dtype)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, causal):
+    """A three-block stack (layer norm, MoDAAttention, MLP, one DepthStream) trained one step on the HIP
+    operator against the same torch modules with the oracle answering every attention call and
+    torch.stack building the cache; then the no-grad path (in-place cache, depth_valid) against it."""
+    import moda_amd
+    from moda_amd import modules
+
+    torch.manual_seed(41)
+    dim, depth, heads, kv_heads, B, N = 256, 3, 4, 2, 2, 70
+    model = moda_amd.MoDAStack(dim, depth, heads, kv_heads, is_causal=causal).to(gpu_device).to(torch.bfloat16)
+    x = (0.5 * torch.randn(B, N, dim, device=gpu_device)).to(torch.bfloat16)
+    w = torch.randn(B, N, dim, device=gpu_device).to(torch.bfloat16)
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        xin = x.clone().requires_grad_(True)
+        y = model(xin)
+        (y.float() * w.float()).sum().backward()
+        return y.detach().float(), xin.grad.float(), {n: p.grad.float().clone() for n, p in model.named_parameters()}
+
+    y_hip, dx_hip, g_hip = step()
+    with torch.no_grad():
+        y_inplace = model(x).float()
+    monkeypatch.setattr(modules, "parallel_moda", _oracle_parallel_moda)
+    monkeypatch.setattr(modules, "stack_depth", lambda layers: oracle.depth_cache_ref(list(layers)))
+    y_ref, dx_ref, g_ref = step()
+
+    def close(a, b, what, tol=3e-2):
+        rel = ((a - b).norm() / b.norm().clamp_min(1e-6)).item()
+        assert rel <= tol, (what, rel)
+
+    close(y_hip, y_ref, "y")
+    close(y_inplace, y_ref, "y (in-place depth cache)")
+    close(dx_hip, dx_ref, "dx")
+    for n in g_ref:
+        close(g_hip[n], g_ref[n], n)
+    # every projection that feeds the depth stream received a gradient through it
+    assert g_hip["blocks.0.attn.kv.weight"].abs().max() > 0
+
+
 def test_empty_and_degenerate(gpu_device):
     import moda_amd
 
