@@ -52,7 +52,7 @@
 extern "C" {
 #endif
 
-#define MODA_HIP_VERSION 102
+#define MODA_HIP_VERSION 103
 
 enum moda_hip_dtype { MODA_HIP_BF16 = 0, MODA_HIP_FP16 = 1, MODA_HIP_FP32 = 2 };
 
@@ -89,7 +89,7 @@ typedef struct moda_hip_desc {
   int64_t T;            /* tokens (key rows)                                       */
   int64_t H;            /* kv heads                                                */
   int64_t G;            /* moda_group_num (folded) or query heads per kv head      */
-  int64_t D;            /* head dim of q/k and of v (must be equal)                */
+  int64_t D;            /* head dim of q, k, kd (and of v, vd, o unless Dv says otherwise) */
   int64_t L;            /* depth slots per token, 0 = no depth stream              */
   int64_t chunk_tokens; /* CHUNK_VISIBLE: base tokens per chunk (C / G), else 0    */
   float scale;          /* logits = scale * <q, key>                               */
@@ -97,6 +97,7 @@ typedef struct moda_hip_desc {
   moda_hip_strides q, k, v, kd, vd, o, d_o, dq, dk, dv, dkd, dvd;
   const int32_t* cu_seqlens; /* packed variable-length batch (see above): DEVICE array of B + 1 offsets, else NULL */
   int64_t total_tokens;      /* with cu_seqlens: cu_seqlens[B], the length of the packed token axis              */
+  int64_t Dv;                /* head dim of v, vd, o, do, dv, dvd; 0 = D.  Dv != D runs on the vector-ALU kernels */
 } moda_hip_desc;
 
 /*

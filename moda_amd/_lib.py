@@ -63,6 +63,7 @@ class Desc(Structure):
         ("dvd", Strides),
         ("cu_seqlens", c_void_p),
         ("total_tokens", c_int64),
+        ("Dv", c_int64),
     ]
 
 

@@ -15,7 +15,7 @@ hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_mfma_probe(const void* operands, int64_t iters, uint64_t* clocks, float* sink, int blocks,
                              hipStream_t stream);
 hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream);
-hipError_t launch_generic(const KArgs& a, int dtype, int D, int which, hipStream_t stream);
+hipError_t launch_generic(const KArgs& a, int dtype, int D, int Dv, int which, hipStream_t stream);
 hipError_t launch_reorg(void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t n_tokens,
                         int64_t row_bytes, void* cache, bool to_cache, hipStream_t stream);
 }  // namespace moda
@@ -38,8 +38,11 @@ bool aligned(const void* p, const moda_hip_strides& s, int esize) {
 // below 16 MiB (tiles have at most 64 rows per pass).
 bool row_stride_ok(const moda_hip_strides& s, int esize) { return s.t >= 0 && s.t * esize < (1ll << 24); }
 
+int value_dim(const moda_hip_desc* d) { return (int)(d->Dv > 0 ? d->Dv : d->D); }
+
 bool use_mfma(const moda_hip_desc* d) {
-  return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && (d->D == 64 || d->D == 128);
+  return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && (d->D == 64 || d->D == 128) &&
+         value_dim(d) == d->D;
 }
 
 // Validates the descriptor and fills the geometry part of KArgs.
@@ -49,6 +52,8 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   if (d->mode < MODA_HIP_CAUSAL || d->mode > MODA_HIP_PLAIN_GQA) return MODA_HIP_EINVAL;
   if (d->B < 0 || d->T < 0 || d->H <= 0 || d->G <= 0 || d->D <= 0 || d->L < 0) return MODA_HIP_EINVAL;
   if (d->D > 256 || d->D % 4 != 0) return MODA_HIP_EUNSUPPORTED;
+  if (d->Dv < 0) return MODA_HIP_EINVAL;
+  if (d->Dv > 256 || d->Dv % 4 != 0) return MODA_HIP_EUNSUPPORTED;
   if (d->mode == MODA_HIP_PLAIN_GQA && d->L != 0) return MODA_HIP_EINVAL;
   if (d->mode == MODA_HIP_DEPTH_ONLY && d->L == 0) return MODA_HIP_EINVAL;
   if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L > 0 && d->chunk_tokens <= 0) return MODA_HIP_EINVAL;
@@ -158,7 +163,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
   a.svd = cvt(d->vd);
   a.so = cvt(d->o);
   hipError_t e = use_mfma(d) ? moda::launch_fwd(a, d->dtype, (int)d->D, (hipStream_t)stream)
-                             : moda::launch_generic(a, d->dtype, (int)d->D, 0, (hipStream_t)stream);
+                             : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 0, (hipStream_t)stream);
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }
 
@@ -255,8 +260,8 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
     if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_dkv(a, d->dtype, (int)d->D, s);
   } else {
     // the generic kernels recompute delta inline; the DELTA stage is a no-op for them
-    if (stages & MODA_HIP_STAGE_DQ) e = moda::launch_generic(a, d->dtype, (int)d->D, 1, s);
-    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_generic(a, d->dtype, (int)d->D, 2, s);
+    if (stages & MODA_HIP_STAGE_DQ) e = moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 1, s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 2, s);
   }
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }

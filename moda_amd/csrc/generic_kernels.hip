@@ -1,5 +1,6 @@
 // Reference-grade kernels for everything the MFMA kernels do not cover: fp32
-// tensors and head dims other than 64/128 (any D <= 256, D % 4 == 0).  Same
+// tensors, head dims other than 64/128 (any D <= 256, D % 4 == 0) and a value
+// head dim Dv that differs from the key head dim D.  Same
 // math, same visible sets and the same base-2 conventions as the MFMA kernels,
 // all arithmetic in fp32 on the vector ALU; one 64-lane wave per query row
 // (forward, dQ) or per key / depth column (dK, dV).  Not tuned: meant for small
@@ -62,7 +63,7 @@ __device__ __forceinline__ bool row_geom(KArgs& a, int64_t gid, RowGeom& g) {
 
 // MODE 0: forward (o, lse).  MODE 1: dq (needs lse; delta computed inline).
 template <typename E, int MODE>
-__global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, const int D) {
+__global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, const int D, const int Dv) {
   __shared__ float qs[4][kMaxD];
   __shared__ float dos[4][kMaxD];
   __shared__ float pb[4][64];
@@ -74,9 +75,9 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, cons
   const int64_t dooff = g.b * a.sdo.b + g.hq * a.sdo.h + (int64_t)g.r * a.sdo.t;
   const int64_t ooff = g.b * a.so.b + g.hq * a.so.h + (int64_t)g.r * a.so.t;
   float delta = 0.f, lse = 0.f;
-  for (int d = lane; d < D; d += 64) {
-    qs[wave][d] = ld<E>(a.q, qoff + d);
-    if (MODE == 1) {
+  for (int d = lane; d < D; d += 64) qs[wave][d] = ld<E>(a.q, qoff + d);
+  if (MODE == 1) {
+    for (int d = lane; d < Dv; d += 64) {
       const float dov = ld<E>(a.d_o, dooff + d);
       dos[wave][d] = dov;
       delta += dov * ld<E>(a.o, ooff + d);
@@ -109,10 +110,9 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, cons
       const bool vis = col < hi;
       float s = 0.f, dp = 0.f;
       if (vis) {
-        for (int d = 0; d < D; d++) {
-          s += qs[wave][d] * ld<E>(kp, kb + (int64_t)col * ks.t + d);
-          if (MODE == 1) dp += dos[wave][d] * ld<E>(vp, vb + (int64_t)col * vs.t + d);
-        }
+        for (int d = 0; d < D; d++) s += qs[wave][d] * ld<E>(kp, kb + (int64_t)col * ks.t + d);
+        if (MODE == 1)
+          for (int d = 0; d < Dv; d++) dp += dos[wave][d] * ld<E>(vp, vb + (int64_t)col * vs.t + d);
       }
       const float s2 = vis ? s * sc : kNegInf;
       float w;  // weight applied to the value / key row of this column
@@ -135,10 +135,11 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, cons
       const void* xp = MODE == 0 ? vp : kp;
       const int64_t xb = MODE == 0 ? vb : kb;
       const int64_t xs = MODE == 0 ? vs.t : ks.t;
+      const int Dx = MODE == 0 ? Dv : D;  // width of the rows being accumulated: values (o) or keys (dq)
 #pragma unroll
       for (int i = 0; i < kDR; i++) {
         const int d = lane + 64 * i;
-        if (d < D) {
+        if (d < Dx) {
           float x = acc[i] * alpha;
           for (int j = 0; j < nc; j++) x += pb[wave][j] * ld<E>(xp, xb + (int64_t)(c0 + j) * xs + d);
           acc[i] = x;
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, cons
 #pragma unroll
     for (int i = 0; i < kDR; i++) {
       const int d = lane + 64 * i;
-      if (d < D) st<E>(a.out_o, ooff + d, acc[i] * inv);
+      if (d < Dv) st<E>(a.out_o, ooff + d, acc[i] * inv);
     }
     if (lane == 0) a.lse[((int64_t)g.b * a.Tq + g.r) * a.Hq + g.hq] = l > 0.f ? m + log2f(l) : kNegInf;
   } else {
@@ -168,7 +169,7 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, cons
 
 // dK/dV: one wave per column (sequence key or depth slot) of one (batch, kv head).
 template <typename E>
-__global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, const int D) {
+__global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, const int D, const int Dv) {
   __shared__ float kc[4][kMaxD];
   __shared__ float vc[4][kMaxD];
   __shared__ float pb[4][64];
@@ -192,10 +193,8 @@ __global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, cons
   const Str3 ks = dep ? a.skd : a.sk, vs = dep ? a.svd : a.sv;
   const int64_t koff = b * ks.b + hkv * ks.h + (int64_t)col * ks.t;
   const int64_t voff = b * vs.b + hkv * vs.h + (int64_t)col * vs.t;
-  for (int d = lane; d < D; d += 64) {
-    kc[wave][d] = ld<E>(kp, koff + d);
-    vc[wave][d] = ld<E>(vp, voff + d);
-  }
+  for (int d = lane; d < D; d += 64) kc[wave][d] = ld<E>(kp, koff + d);
+  for (int d = lane; d < Dv; d += 64) vc[wave][d] = ld<E>(vp, voff + d);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -221,9 +220,9 @@ __global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, cons
       float p = 0.f, ds = 0.f;
       if (r < qhi) {
         float s = 0.f, dp = 0.f, delta = 0.f;
-        for (int d = 0; d < D; d++) {
+        for (int d = 0; d < D; d++) s += kc[wave][d] * ld<E>(a.q, qb + (int64_t)r * a.sq.t + d);
+        for (int d = 0; d < Dv; d++) {
           const float dov = ld<E>(a.d_o, dob + (int64_t)r * a.sdo.t + d);
-          s += kc[wave][d] * ld<E>(a.q, qb + (int64_t)r * a.sq.t + d);
           dp += vc[wave][d] * dov;
           delta += dov * ld<E>(a.o, ob + (int64_t)r * a.so.t + d);
         }
@@ -240,12 +239,13 @@ __global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, cons
       for (int i = 0; i < kDR; i++) {
         const int d = lane + 64 * i;
         if (d < D) {
-          float xk = dk[i], xv = dv[i];
-          for (int j = 0; j < nr; j++) {
-            xk += dsb[wave][j] * ld<E>(a.q, qb + (int64_t)(r0 + j) * a.sq.t + d);
-            xv += pb[wave][j] * ld<E>(a.d_o, dob + (int64_t)(r0 + j) * a.sdo.t + d);
-          }
+          float xk = dk[i];
+          for (int j = 0; j < nr; j++) xk += dsb[wave][j] * ld<E>(a.q, qb + (int64_t)(r0 + j) * a.sq.t + d);
           dk[i] = xk;
+        }
+        if (d < Dv) {
+          float xv = dv[i];
+          for (int j = 0; j < nr; j++) xv += pb[wave][j] * ld<E>(a.d_o, dob + (int64_t)(r0 + j) * a.sdo.t + d);
           dv[i] = xv;
         }
       }
@@ -261,37 +261,35 @@ __global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, cons
 #pragma unroll
   for (int i = 0; i < kDR; i++) {
     const int d = lane + 64 * i;
-    if (d < D) {
-      st<E>(dkp, dkoff + d, dk[i] * a.scale);
-      st<E>(dvp, dvoff + d, dv[i]);
-    }
+    if (d < D) st<E>(dkp, dkoff + d, dk[i] * a.scale);
+    if (d < Dv) st<E>(dvp, dvoff + d, dv[i]);
   }
 }
 
 template <typename E>
-hipError_t launch_generic_t(const KArgs& a, int D, int which, hipStream_t stream) {
+hipError_t launch_generic_t(const KArgs& a, int D, int Dv, int which, hipStream_t stream) {
   if (which == 0 || which == 1) {
     const int64_t rows = (int64_t)a.B * a.Hq * a.Tq;
     if (rows == 0) return hipSuccess;
     const unsigned nblk = (unsigned)((rows + 3) / 4);
     if (which == 0)
-      hipLaunchKernelGGL((generic_row_kernel<E, 0>), dim3(nblk), dim3(256), 0, stream, a, D);
+      hipLaunchKernelGGL((generic_row_kernel<E, 0>), dim3(nblk), dim3(256), 0, stream, a, D, Dv);
     else
-      hipLaunchKernelGGL((generic_row_kernel<E, 1>), dim3(nblk), dim3(256), 0, stream, a, D);
+      hipLaunchKernelGGL((generic_row_kernel<E, 1>), dim3(nblk), dim3(256), 0, stream, a, D, Dv);
   } else {
     const int64_t ncol = (int64_t)(a.has_seq ? a.T : 0) + (int64_t)a.T * a.L;
     const int64_t cols = ncol * a.B * a.Hkv;
     if (cols == 0) return hipSuccess;
-    hipLaunchKernelGGL((generic_col_kernel<E>), dim3((unsigned)((cols + 3) / 4)), dim3(256), 0, stream, a, D);
+    hipLaunchKernelGGL((generic_col_kernel<E>), dim3((unsigned)((cols + 3) / 4)), dim3(256), 0, stream, a, D, Dv);
   }
   return hipGetLastError();
 }
 
 // which: 0 forward, 1 dq, 2 dk/dv
-hipError_t launch_generic(const KArgs& a, int dtype, int D, int which, hipStream_t stream) {
-  if (dtype == 0) return launch_generic_t<__bf16>(a, D, which, stream);
-  if (dtype == 1) return launch_generic_t<_Float16>(a, D, which, stream);
-  if (dtype == 2) return launch_generic_t<float>(a, D, which, stream);
+hipError_t launch_generic(const KArgs& a, int dtype, int D, int Dv, int which, hipStream_t stream) {
+  if (dtype == 0) return launch_generic_t<__bf16>(a, D, Dv, which, stream);
+  if (dtype == 1) return launch_generic_t<_Float16>(a, D, Dv, which, stream);
+  if (dtype == 2) return launch_generic_t<float>(a, D, Dv, which, stream);
   return hipErrorInvalidValue;
 }
 

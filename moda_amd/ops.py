@@ -115,6 +115,8 @@ def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=
     d.H = src.shape[2]
     d.G = G
     d.D = q.shape[3]
+    val = vd if mode == _lib.DEPTH_ONLY else v
+    d.Dv = val.shape[3]
     d.L = L
     if depth_valid is not None and L > 0:
         assert 1 <= depth_valid <= L, f"depth_valid must be in [1, {L}], got {depth_valid}"
@@ -157,8 +159,6 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None, 
     if kd is not None and T == 0:
         L = 0
     val = vd if mode == _lib.DEPTH_ONLY else v
-    if val.shape[-1] != q.shape[-1]:
-        raise NotImplementedError("value head dim must equal key head dim")
     o = torch.empty(q.shape[0], q.shape[1], q.shape[2], val.shape[-1], dtype=val.dtype, device=q.device)
     lse = torch.empty(q.shape[0], q.shape[1], q.shape[2], dtype=torch.float32, device=q.device)
     if L == 0:

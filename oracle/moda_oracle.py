@@ -471,21 +471,23 @@ def depth_cache_grad_ref(dcache: torch.Tensor, L: int):
 # seeded inputs, metrics, algorithmic work
 # --------------------------------------------------------------------------
 def make_inputs(B, T, H, D, L, G=1, seed=0, dtype=torch.float32, std=1.0, do_std=1.0,
-                prescale_q=False, depth_only=False, Hq=None):
+                prescale_q=False, depth_only=False, Hq=None, Dv=None):
     """Deterministic inputs from a CPU generator, drawn in fp32 in the order
     q, k, v, kd, vd, do and then cast.  ``Hq`` (plain GQA layout) makes q
-    ``[B,T,Hq,D]`` instead of the folded ``[B,T*G,H,D]``."""
+    ``[B,T,Hq,D]`` instead of the folded ``[B,T*G,H,D]``; ``Dv`` gives v, vd and do a
+    head dim of their own."""
     gen = torch.Generator().manual_seed(seed)
     rn = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
     qshape = (B, T, Hq, D) if Hq is not None else (B, T * G, H, D)
+    Dv = D if Dv is None else Dv
     q = rn(*qshape) * std
     if prescale_q:
         q = q * (D ** -0.5)
     k = rn(B, T, H, D) * std
-    v = rn(B, T, H, D) * std
+    v = rn(B, T, H, Dv) * std
     kd = rn(B, T * L, H, D) * std if L > 0 else None
-    vd = rn(B, T * L, H, D) * std if L > 0 else None
-    do = rn(*qshape) * do_std
+    vd = rn(B, T * L, H, Dv) * std if L > 0 else None
+    do = rn(*qshape[:3], Dv) * do_std
     c = lambda x: None if x is None else x.to(dtype)
     out = {"q": c(q), "k": c(k), "v": c(v), "kd": c(kd), "vd": c(vd), "do": c(do)}
     if depth_only:

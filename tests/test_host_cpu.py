@@ -32,8 +32,8 @@ def test_descriptor_layout_and_version():
     from moda_amd import _lib
 
     lib = _lib.load()
-    assert lib.moda_hip_version() == 102
-    assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24 + 16
+    assert lib.moda_hip_version() == 103
+    assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24 + 24
     assert _lib.Desc.cu_seqlens.offset == 80 + 12 * 24
     assert _lib.Desc.q.offset == 80
     # a descriptor with the wrong struct_size is rejected without touching any device
@@ -77,6 +77,10 @@ def test_descriptor_validation_codes():
     assert lib.moda_hip_fwd(ctypes.byref(desc(mode=_lib.DEPTH_ONLY)), null, null, null, null, null, null, null, null) == -1
     assert lib.moda_hip_fwd(ctypes.byref(desc(mode=_lib.PLAIN_GQA, L=2)), null, null, null, null, null, null, null, null) == -1
     assert lib.moda_hip_fwd(ctypes.byref(desc(mode=_lib.CHUNK_VISIBLE, L=2)), null, null, null, null, null, null, null, null) == -1
+    # value head dim: negative is invalid, beyond 256 or not a multiple of 4 unsupported
+    assert lib.moda_hip_fwd(ctypes.byref(desc(Dv=-4)), null, null, null, null, null, null, null, null) == -1
+    assert lib.moda_hip_fwd(ctypes.byref(desc(Dv=512)), null, null, null, null, null, null, null, null) == -2
+    assert lib.moda_hip_fwd(ctypes.byref(desc(Dv=30)), null, null, null, null, null, null, null, null) == -2
     # empty problem is a successful no-op
     assert lib.moda_hip_fwd(ctypes.byref(desc(T=0)), null, null, null, null, null, null, null, null) == 0
     # misaligned pointer (never dereferenced: alignment is checked first)

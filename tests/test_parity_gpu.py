@@ -603,6 +603,33 @@ def test_mfma_probe_runs(gpu_device):
 
 
 # ---------------------------------------------------------------------------
+# value head dim different from the key head dim (o [B, T*G, H, V], moda_v14.py:2792-2815)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("case", [
+    (2, 70, 2, 64, 128, 3, 2, "causal", 0, torch.bfloat16),
+    (1, 130, 1, 128, 64, 5, 4, "noncausal", 0, torch.float16),
+    (1, 50, 2, 32, 96, 2, 1, "chunk_visible", 8, torch.float32),
+    (1, 40, 2, 64, 32, 4, 2, "depth_only", 0, torch.bfloat16),
+    (1, 33, 1, 96, 256, 0, 2, "causal", 0, torch.bfloat16),
+], ids=lambda c: f"{c[7]}-D{c[3]}-Dv{c[4]}")
+def test_value_head_dim_differs_from_key_head_dim(gpu_device, case):
+    import moda_amd
+
+    B, T, H, D, Dv, L, G, mode, cb, dtype = case
+    say(f"[Dv] {case}")
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=43, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"), Dv=Dv)
+    sc = D ** -0.5
+    ref = oracle.moda_dense_fwd_bwd(inp, sc, G, mode, cb)
+    got = run_hip(to_dev(inp, gpu_device), sc, G, mode, cb)
+    assert got["o"].shape[-1] == Dv and got["dq"].shape[-1] == D
+    compare_all(got, ref, dtype, str(case))
+    if mode == "causal":  # and through the public interface
+        dev = to_dev(inp, gpu_device)
+        o = moda_amd.parallel_moda(dev["q"], dev["k"], dev["v"], cached_k=dev["kd"], cached_v=dev["vd"], moda_group_num=G)
+        check("o", o, ref["o"], dtype, "public " + str(case))
+
+
+# ---------------------------------------------------------------------------
 # packed variable-length batches (cu_seqlens): the oracle evaluates every sequence on its own
 # ---------------------------------------------------------------------------
 PACKED = [
