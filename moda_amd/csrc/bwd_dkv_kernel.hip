@@ -469,6 +469,7 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   const int64_t n_seq_tiles = a.has_seq ? (a.T + 127) / 128 : 0;
   const int64_t n_dep_tiles = (a.L > 0 && !depth_by_columns) ? ((int64_t)a.T * a.L + 127) / 128 : 0;
   const int64_t nblk = (n_seq_tiles + n_dep_tiles) * a.B * a.Hkv;
+  if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   if (nblk > 0) {
     if (a.cu)
       hipLaunchKernelGGL((dkv_kernel<T, HD, true>), dim3((unsigned)nblk), dim3(512), smem, stream, a);

@@ -21,12 +21,15 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a_in) {
   constexpr int TPR = HD / 8;         // threads per row
   constexpr int RPB = 256 / TPR;      // rows per block
   const int tid = threadIdx.x;
-  const int bh = blockIdx.y;
+  // one-dimensional grid (row blocks of the longest sequence x batch*heads): the y extent of a grid stops at 65535
+  const int nrb = (a_in.Tq + RPB - 1) / RPB;
+  const int bh = blockIdx.x / nrb;
+  const int rb = blockIdx.x - bh * nrb;
   KArgs a = a_in;
   int b = bh / a.Hq;
   const int hq = bh % a.Hq;
   enter_sequence(a, b);
-  const int r = blockIdx.x * RPB + tid / TPR;
+  const int r = rb * RPB + tid / TPR;
   const int c = (tid % TPR) * 8;
   float acc = 0.f;
   if (r < a.Tq) {
@@ -250,7 +253,9 @@ template <typename T, int HD>
 hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
   if (a.Tq == 0 || a.B * a.Hq == 0) return hipSuccess;
   constexpr int RPB = 256 / (HD / 8);
-  hipLaunchKernelGGL((delta_kernel<T, HD>), dim3((a.Tq + RPB - 1) / RPB, a.B * a.Hq), dim3(256), 0, stream, a);
+  const int64_t nblk = (int64_t)((a.Tq + RPB - 1) / RPB) * a.B * a.Hq;
+  if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((delta_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 
@@ -262,6 +267,7 @@ hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
   if (ea != hipSuccess) return ea;
   const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
+  if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   hipLaunchKernelGGL((dq_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
   return hipGetLastError();
 }

@@ -278,6 +278,7 @@ hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
   if (ea != hipSuccess) return ea;
   const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
+  if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   hipLaunchKernelGGL((fwd_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
   return hipGetLastError();
 }

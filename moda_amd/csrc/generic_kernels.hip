@@ -271,6 +271,7 @@ hipError_t launch_generic_t(const KArgs& a, int D, int Dv, int which, hipStream_
   if (which == 0 || which == 1) {
     const int64_t rows = (int64_t)a.B * a.Hq * a.Tq;
     if (rows == 0) return hipSuccess;
+    if ((rows + 3) / 4 >= (1ll << 31)) return hipErrorInvalidValue;
     const unsigned nblk = (unsigned)((rows + 3) / 4);
     if (which == 0)
       hipLaunchKernelGGL((generic_row_kernel<E, 0>), dim3(nblk), dim3(256), 0, stream, a, D, Dv);
@@ -280,6 +281,7 @@ hipError_t launch_generic_t(const KArgs& a, int D, int Dv, int which, hipStream_
     const int64_t ncol = (int64_t)(a.has_seq ? a.T : 0) + (int64_t)a.T * a.L;
     const int64_t cols = ncol * a.B * a.Hkv;
     if (cols == 0) return hipSuccess;
+    if ((cols + 3) / 4 >= (1ll << 31)) return hipErrorInvalidValue;
     hipLaunchKernelGGL((generic_col_kernel<E>), dim3((unsigned)((cols + 3) / 4)), dim3(256), 0, stream, a, D, Dv);
   }
   return hipGetLastError();

@@ -772,6 +772,15 @@ def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, causal):
     assert g_hip["blocks.0.attn.kv.weight"].abs().max() > 0
 
 
+def test_more_than_65535_batch_heads(gpu_device):
+    """Launch grids are one-dimensional: batch x heads beyond the 65535 limit of a grid's y extent."""
+    B, T, H, D, L, G = 70000, 3, 1, 64, 2, 2
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=47, dtype=torch.bfloat16, std=0.5)
+    ref = oracle.moda_dense_fwd_bwd(inp, D ** -0.5, G, "causal")
+    got = run_hip(to_dev(inp, gpu_device), D ** -0.5, G, "causal")
+    compare_all(got, ref, torch.bfloat16, "many batch-heads")
+
+
 def test_empty_and_degenerate(gpu_device):
     import moda_amd
 
