@@ -772,6 +772,66 @@ def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, causal):
     assert g_hip["blocks.0.attn.kv.weight"].abs().max() > 0
 
 
+# ---------------------------------------------------------------------------
+# seeded random sweep over shapes, modes and options (ragged sizes, every option combined)
+# ---------------------------------------------------------------------------
+def _random_case(seed):
+    import random
+
+    rnd = random.Random(seed)
+    mode = rnd.choice(["causal", "causal", "noncausal", "chunk_visible", "depth_only"])
+    D = rnd.choice([64, 128])
+    G = rnd.choice([1, 2, 4, 8])
+    H = rnd.choice([1, 2, 3])
+    L = rnd.choice([0, 1, 2, 3, 5, 9]) if mode != "depth_only" else rnd.choice([1, 2, 5, 9])
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    packed = rnd.random() < 0.4
+    if packed:
+        lengths = [rnd.choice([0, 1, 2, 17, 63, 64, 65, 130, 257]) for _ in range(rnd.randint(1, 4))]
+        if sum(lengths) == 0:
+            lengths[0] = 33
+        B = 1
+    else:
+        lengths = [rnd.choice([1, 2, 3, 31, 64, 65, 127, 129, 200, 301])]
+        B = rnd.choice([1, 2])
+    cb = rnd.choice([1, 2, 16, 64 // G if 64 // G > 0 else 1]) if mode == "chunk_visible" else 0
+    valid = None
+    if L > 1 and mode != "chunk_visible" and rnd.random() < 0.4:
+        valid = rnd.randint(1, L)
+    return mode, D, G, H, L, dtype, packed, lengths, B, cb, valid
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_sweep(gpu_device, seed):
+    from moda_amd import ops
+
+    mode, D, G, H, L, dtype, packed, lengths, B, cb, valid = _random_case(1000 + seed)
+    say(f"[sweep {seed}] mode={mode} D={D} G={G} H={H} L={L} {dtype} packed={packed} lengths={lengths} B={B} cb={cb} valid={valid}")
+    total = sum(lengths)
+    inp = oracle.make_inputs(B, total, H, D, L, G, seed=seed, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
+    sc = D ** -0.5
+    ref_inp = dict(inp)
+    if valid is not None:
+        ref_inp["kd"] = oracle.compact_depth(inp["kd"], total, valid)
+        ref_inp["vd"] = oracle.compact_depth(inp["vd"], total, valid)
+    cu = _cu(lengths)
+    if packed:
+        ref = oracle.moda_packed_fwd_bwd(ref_inp, cu, sc, G, mode, cb)
+    else:
+        ref = oracle.moda_dense_fwd_bwd(ref_inp, sc, G, mode, cb)
+    if valid is not None:
+        ref["dkd"] = oracle.scatter_depth_grad(ref["dkd"], total, L)
+        ref["dvd"] = oracle.scatter_depth_grad(ref["dvd"], total, L)
+    dev = to_dev(inp, gpu_device)
+    pk = ops._packed(torch.tensor(cu, device=gpu_device), dev["q"], G) if packed else None
+    m = MODE_ID[mode]
+    o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], sc, G, cb, depth_valid=valid, packed=pk)
+    dq, dk, dv, dkd, dvd = ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], o, lse, dev["do"], sc, G,
+                                        cb, depth_valid=valid, packed=pk)
+    got = {"o": o, "lse": lse, "dq": dq, "dk": dk, "dv": dv, "dkd": dkd, "dvd": dvd}
+    compare_all(got, ref, dtype, f"sweep {seed}")
+
+
 def test_more_than_65535_batch_heads(gpu_device):
     """Launch grids are one-dimensional: batch x heads beyond the 65535 limit of a grid's y extent."""
     B, T, H, D, L, G = 70000, 3, 1, 64, 2, 2
