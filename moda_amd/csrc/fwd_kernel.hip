@@ -23,13 +23,18 @@
 
 namespace moda {
 
+// launch shape of the forward kernel for all but small problems
+using FwdLarge = RowLargePP;
+
 // ADDR bit 0: a (batch, head) slice is wider than 2 GiB (descriptors anchored per tile instead of 32-bit
 // offsets inside the slice); bit 1: packed variable-length batch
 template <typename T, int HD, typename Shape, int ADDR>
 __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in) {
   constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST,
                 DIST = Shape::DIST;
-  static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
+  constexpr bool PP = Shape::PP;
+  static_assert(NST >= DIST + 1 + (PP ? 1 : 0) && DIST >= 1 && DIST <= 2,
+                "ring must hold the tile in use, the tiles in flight and (ping-pong) the previous tile");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
@@ -156,14 +161,15 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   __syncthreads();
   int c_st = 0;  // ring stage of the tile being consumed
 
-  // one column tile: S^T = K Q^T, online softmax, O^T += V^T P^T
-  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, int lo, int hi) {
+  // One column tile in two halves.  front: S^T = K Q^T and the online softmax, leaving the rounded
+  // probabilities in P; back: O^T += V^T P^T.
+  i32x4 P[4];
+  TrPipe<T, HD, 4, 2> pv;
+  auto front = [&](auto masked, lds_cptr Kc, int col0, int lo, int hi, auto&& after_scores) {
     constexpr bool MASKED = decltype(masked)::value;
     f32x16 s[2];
     mfma_rows<T, HD, 2, 4>(oa, Kc, Qr, s);
-    // first V^T operands start travelling while the softmax runs
-    TrPipe<T, HD, 4, 2> pv;
-    pv.prefetch(oa, Vc);
+    after_scores();
     // row maximum of the raw scores (scale > 0, so it commutes with the max)
     float mx = kNegInf;
 #pragma unroll
@@ -208,50 +214,122 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         else
           rs0 += p;
       }
-    i32x4 P[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
     l += pair_sum(rs0 + rs1);
+  };
+  // the whole tile at once: the first V^T operands start travelling while the softmax runs
+  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, int lo, int hi) {
+    front(masked, Kc, col0, lo, hi, [&]() { pv.prefetch(oa, Vc); });
     pv.run(oa, Vc, P, o);
   };
-
-  // phase 1: tiles fully visible to every row -- no masks, no visibility tests.  The loop is unrolled
-  // over the ring stages so that each copy reads its tile at a compile-time LDS offset (the stage
-  // offset then rides in the instructions' immediate field instead of costing an address add per
-  // operand read); the remainder runs the same body with the stage in a register.
-  int it = 0;
-  auto full_tile = [&](lds_cptr Kc) {
-    if (it + DIST < ntiles) issue(it + DIST);
-    tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, 0, 0);
-    wait_tile(it + 1);
-    __syncthreads();
-    it++;
+  auto back = [&](lds_cptr Vc) {
+    pv.prefetch(oa, Vc);
+    pv.run(oa, Vc, P, o);
   };
-  for (; it + NST <= n_full;) {
-    full_tile(smem);
-    full_tile(smem + 1 * 2 * BN * HD);
-    if (NST > 2) full_tile(smem + 2 * 2 * BN * HD);
-  }
-  c_st = 0;
-  for (; it < n_full;) {
-    full_tile(smem + c_st * 2 * BN * HD);
-    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
-  }
-  // phase 2: boundary sequence tiles and depth tiles
-  for (; it < ntiles; it++) {
-    if (it + DIST < ntiles) issue(it + DIST);
-    const bool dep = it >= n_seq;
-    const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
-    const int lo = dep ? dlo : 0;
-    const int hi = dep ? dhi : shi;
-    const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
-    if (__any(touches)) {
-      lds_cptr Kc = smem + c_st * 2 * BN * HD;
-      tile(std::true_type{}, Kc, Kc + BN * HD, col0, lo, hi);
+  auto stage_k = [&](int st) { return smem + st * 2 * BN * HD; };
+
+  // Ping-pong: the two waves of a SIMD (wave w and w + W/2) would otherwise run the same phase at the
+  // same time -- matrix pipe contended during the MFMA phases, idle during both softmaxes.  The upper
+  // half of the workgroup therefore runs half a tile behind: between two barriers it first finishes the
+  // previous tile (V product), then does scores and softmax of the current one, so its softmax overlaps
+  // the lower half's V product and its V product the lower half's scores.  The previous tile's V must
+  // survive one more barrier interval, hence the extra ring stage.
+  const bool late = PP && __builtin_amdgcn_readfirstlane(wave) >= Shape::W / 2;
+  int it = 0;
+  if (!late) {
+    // phase 1: tiles fully visible to every row -- no masks, no visibility tests.  The loop is unrolled
+    // over the ring stages so that each copy reads its tile at a compile-time LDS offset (the stage
+    // offset then rides in the instructions' immediate field instead of costing an address add per
+    // operand read); the remainder runs the same body with the stage in a register.
+    auto full_tile = [&](lds_cptr Kc) {
+      if (it + DIST < ntiles) issue(it + DIST);
+      tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, 0, 0);
+      wait_tile(it + 1);
+      __syncthreads();
+      it++;
+    };
+    for (; it + NST <= n_full;) {
+      full_tile(smem);
+      full_tile(smem + 1 * 2 * BN * HD);
+      if (NST > 2) full_tile(smem + 2 * 2 * BN * HD);
+      if (NST > 3) full_tile(smem + 3 * 2 * BN * HD);
     }
-    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
-    wait_tile(it + 1);
-    __syncthreads();
+    c_st = 0;
+    for (; it < n_full;) {
+      full_tile(stage_k(c_st));
+      c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    }
+    // phase 2: boundary sequence tiles and depth tiles
+    for (; it < ntiles; it++) {
+      if (it + DIST < ntiles) issue(it + DIST);
+      const bool dep = it >= n_seq;
+      const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
+      const int lo = dep ? dlo : 0;
+      const int hi = dep ? dhi : shi;
+      const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
+      if (__any(touches)) {
+        lds_cptr Kc = stage_k(c_st);
+        tile(std::true_type{}, Kc, Kc + BN * HD, col0, lo, hi);
+      }
+      c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+      wait_tile(it + 1);
+      __syncthreads();
+    }
+  } else {
+    // the late half: [V product of the previous tile] [scores + softmax of this tile] [barrier]
+    if (n_full > 0) {  // first tile: nothing to finish yet
+      if (DIST < ntiles) issue(DIST);
+      front(std::false_type{}, smem, 0, 0, 0, []() {});
+      wait_tile(1);
+      __syncthreads();
+      it = 1;
+    }
+    // `Vp`: V tile of the previous tile, `Kc`: K tile of this one
+    auto full_tile = [&](lds_cptr Vp, lds_cptr Kc) {
+      if (it + DIST < ntiles) issue(it + DIST);
+      back(Vp);
+      front(std::false_type{}, Kc, it * BN, 0, 0, []() {});
+      wait_tile(it + 1);
+      __syncthreads();
+      it++;
+    };
+    if (NST == 4) {
+      // it % NST == 1 here (or no full tile at all): copies with compile-time stages
+      for (; it + NST <= n_full;) {
+        full_tile(smem + BN * HD, smem + 1 * 2 * BN * HD);
+        full_tile(smem + 1 * 2 * BN * HD + BN * HD, smem + 2 * 2 * BN * HD);
+        full_tile(smem + 2 * 2 * BN * HD + BN * HD, smem + 3 * 2 * BN * HD);
+        full_tile(smem + 3 * 2 * BN * HD + BN * HD, smem);
+      }
+    }
+    c_st = it % NST;
+    for (; it < n_full;) {
+      const int prev = (c_st == 0) ? NST - 1 : c_st - 1;
+      full_tile(stage_k(prev) + BN * HD, stage_k(c_st));
+      c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    }
+    bool pending = it > 0;  // a tile whose V product is still to do
+    int p_st = (c_st == 0) ? NST - 1 : c_st - 1;
+    for (; it < ntiles; it++) {
+      if (it + DIST < ntiles) issue(it + DIST);
+      if (pending) back(stage_k(p_st) + BN * HD);
+      pending = false;
+      const bool dep = it >= n_seq;
+      const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
+      const int lo = dep ? dlo : 0;
+      const int hi = dep ? dhi : shi;
+      const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
+      if (__any(touches)) {
+        front(std::true_type{}, stage_k(c_st), col0, lo, hi, []() {});
+        pending = true;
+        p_st = c_st;
+      }
+      c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+      wait_tile(it + 1);
+      __syncthreads();
+    }
+    if (pending) back(stage_k(p_st) + BN * HD);
   }
 
   if (valid) {
@@ -291,38 +369,38 @@ hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
   const bool wide = span > 0x7fffffffll;
   const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
   if (a.cu) {
-    if (wide) return launch_fwd_t_shape<T, HD, RowLarge, 3>(a, stream);
+    if (wide) return launch_fwd_t_shape<T, HD, FwdLarge, 3>(a, stream);
     if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, 2>(a, stream);
-    return launch_fwd_t_shape<T, HD, RowLarge, 2>(a, stream);
+    return launch_fwd_t_shape<T, HD, FwdLarge, 2>(a, stream);
   }
-  if (wide) return launch_fwd_t_shape<T, HD, RowLarge, 1>(a, stream);
+  if (wide) return launch_fwd_t_shape<T, HD, FwdLarge, 1>(a, stream);
   if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, 0>(a, stream);
-  return launch_fwd_t_shape<T, HD, RowLarge, 0>(a, stream);
+  return launch_fwd_t_shape<T, HD, FwdLarge, 0>(a, stream);
 }
 
-template __global__ void fwd_kernel<BF16, 128, RowLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowLarge, 1>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowLarge, 1>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowLarge, 1>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, FwdLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, FwdLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, FwdLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, FwdLarge, 0>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, FwdLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, FwdLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, FwdLarge, 1>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, FwdLarge, 1>(const KArgs);
 template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, 0>(const KArgs);
 template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, 0>(const KArgs);
 template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, 0>(const KArgs);
 template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, 0>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowLarge, 3>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, FwdLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<BF16, 128, FwdLarge, 3>(const KArgs);
 template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, 2>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowLarge, 3>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, FwdLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<BF16, 64, FwdLarge, 3>(const KArgs);
 template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowLarge, 3>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, FwdLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<FP16, 128, FwdLarge, 3>(const KArgs);
 template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowLarge, 3>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, FwdLarge, 2>(const KArgs);
+template __global__ void fwd_kernel<FP16, 64, FwdLarge, 3>(const KArgs);
 template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, 2>(const KArgs);
 
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream) {

@@ -14,16 +14,25 @@ namespace moda {
 // of 16 rows per pass (the LDS swizzle repeats every 16 rows).
 struct RowLarge {
   static constexpr int W = 8, NST = 3, DIST = 2;
+  static constexpr bool PP = false;
+};
+// RowLarge with the upper half of the workgroup running half a tile behind the lower half (see the
+// forward kernel); one more ring stage keeps the previous tile's V alive for it.
+struct RowLargePP {
+  static constexpr int W = 8, NST = 4, DIST = 2;
+  static constexpr bool PP = true;
 };
 template <int HD>
 struct RowSmall;
 template <>
 struct RowSmall<64> {
   static constexpr int W = 2, NST = 3, DIST = 2;  // 48 KB of LDS: three workgroups per compute unit
+  static constexpr bool PP = false;
 };
 template <>
 struct RowSmall<128> {
   static constexpr int W = 4, NST = 2, DIST = 1;  // 64 KB of LDS: two workgroups per compute unit
+  static constexpr bool PP = false;
 };
 
 // Host side: the small shape is used when the large one would not even give every compute unit

@@ -773,6 +773,30 @@ def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, causal):
 
 
 # ---------------------------------------------------------------------------
+# the throughput launch shape (256-row workgroups, ping-pong halves) on short and ragged sequences: enough
+# (batch, head) pairs that the small-problem shape is not chosen
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("case", [
+    (64, 1, 8, 64, 2, 1, "causal", 0, torch.bfloat16),
+    (64, 63, 8, 64, 0, 1, "causal", 0, torch.bfloat16),
+    (64, 130, 8, 64, 3, 2, "causal", 0, torch.float16),
+    (32, 300, 16, 128, 5, 4, "noncausal", 0, torch.bfloat16),
+    (64, 129, 8, 128, 2, 2, "chunk_visible", 16, torch.bfloat16),
+    (64, 65, 8, 128, 7, 4, "depth_only", 0, torch.float16),
+    (128, 257, 4, 64, 1, 1, "causal", 0, torch.bfloat16),
+], ids=lambda c: f"{c[6]}-B{c[0]}-T{c[1]}-D{c[3]}-L{c[4]}-G{c[5]}")
+def test_large_launch_shape_on_ragged_inputs(gpu_device, case):
+    B, T, H, D, L, G, mode, cb, dtype = case
+    say(f"[large shape] {case}")
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=53, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
+    sc = D ** -0.5
+    dev = to_dev(inp, gpu_device)
+    got = run_hip(dev, sc, G, mode, cb)
+    ref = oracle.moda_dense_fwd_bwd(dev, sc, G, mode, cb)  # the oracle's dense form, evaluated on the device
+    compare_all(got, ref, dtype, str(case))
+
+
+# ---------------------------------------------------------------------------
 # seeded random sweep over shapes, modes and options (ragged sizes, every option combined)
 # ---------------------------------------------------------------------------
 def _random_case(seed):
