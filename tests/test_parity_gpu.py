@@ -797,6 +797,43 @@ def test_large_launch_shape_on_ragged_inputs(gpu_device, case):
 
 
 # ---------------------------------------------------------------------------
+# peaked softmax: logits of several dozen (base 2), where the lazily moved exponent reference, the
+# 2^8 head room of the rounded probabilities and the fp16 range are all in play
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("case", [
+    (1, 300, 2, 128, 4, 2, "causal", torch.bfloat16, 3.0),
+    (1, 300, 2, 64, 4, 2, "causal", torch.float16, 3.0),
+    (2, 200, 2, 128, 3, 4, "noncausal", torch.bfloat16, 4.0),
+    (64, 130, 8, 64, 3, 2, "causal", torch.bfloat16, 3.0),
+    (1, 257, 1, 128, 6, 1, "depth_only", torch.float16, 3.0),
+    (1, 1000, 1, 128, 2, 1, "causal", torch.bfloat16, 6.0),
+], ids=lambda c: f"{c[6]}-T{c[1]}-D{c[3]}-std{c[8]}-{str(c[7])[6:]}")
+def test_peaked_softmax(gpu_device, case):
+    B, T, H, D, L, G, mode, dtype, std = case
+    say(f"[peaked] {case}")
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=5, dtype=dtype, std=std, depth_only=(mode == "depth_only"))
+    for n in ("v", "vd"):  # values stay of order one: the test is about the softmax
+        if inp[n] is not None:
+            inp[n] = (inp[n].float() / std).to(dtype)
+    dev = to_dev(inp, gpu_device)
+    got = run_hip(dev, D ** -0.5, G, mode)
+    ref = oracle.moda_dense_fwd_bwd(dev, D ** -0.5, G, mode)
+    assert ref["lse"].abs().max() > 40  # the case is what it claims to be
+    # Gradients here are sums of terms of order ten that cancel; P and dS are rounded to the 16-bit input
+    # type before the second product (as in the reference, moda_v14.py:209, 712), so the error of an
+    # element scales with the tensor's magnitude, not with the element's: bound it by atol + rtol * max|ref|.
+    atol, rtol = TOL[dtype]
+    for n in ("o", "dq", "dk", "dv", "dkd", "dvd"):
+        if ref[n] is None:
+            continue
+        g, r = got[n].float(), ref[n].float()
+        assert torch.isfinite(g).all(), n
+        bound = atol + rtol * r.abs().max().item()
+        assert (g - r).abs().max().item() <= bound, (n, (g - r).abs().max().item(), bound)
+    check("lse", got["lse"], ref["lse"], dtype, str(case))
+
+
+# ---------------------------------------------------------------------------
 # seeded random sweep over shapes, modes and options (ragged sizes, every option combined)
 # ---------------------------------------------------------------------------
 def _random_case(seed):
