@@ -182,11 +182,16 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   __syncthreads();
   int c_st = 0;  // ring stage of the tile being consumed
 
+  // start value of every dP^T accumulator block: this lane's row constant -rowsum(o * do), so that the
+  // subtraction costs no instruction per element
+  f32x16 dp_init;
+#pragma unroll
+  for (int i = 0; i < 16; i++) dp_init[i] = delta;
   // one column tile: S^T = K Q^T and dP^T = V dO^T in one MFMA pipeline, dS^T, dQ^T += K^T dS^T
   auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, int lo, int hi) {
     constexpr bool MASKED = decltype(masked)::value;
     f32x16 s[2], dp[2];
-    mfma_rows2<T, HD, 2, 4>(oa, Kc, Qr, s, Vc, dOr, dp);
+    mfma_rows2<T, HD, 2, 4>(oa, Kc, Qr, s, Vc, dOr, dp, dp_init);
     TrPipe<T, HD, 4, 2> kt;
     kt.prefetch(oa, Kc);
 #pragma unroll
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
           const int c = col0 + 32 * bb + acc_row(i, g);
           p = (c >= lo && c < hi) ? p : 0.f;
         }
-        s[bb][i] = p * (dp[bb][i] + delta);  // delta holds minus rowsum(o * do)
+        s[bb][i] = p * dp[bb][i];  // dp started from minus rowsum(o * do)
       }
     i32x4 DS[4];
 #pragma unroll
