@@ -356,8 +356,8 @@ def main():
     # figures are recorded here per workload and kernel; a workload without a recorded run reports null.
     GiB = float(1 << 30)
     measured_hbm_bytes = {
-        # the dK/dV stage at c4 is two launches: dkv_kernel (17.17 GiB) and depth_cols_kernel (7.04 GiB)
-        ("c4", "fwd_kernel"): 5.74 * GiB, ("c4", "dq_kernel"): 5.97 * GiB, ("c4", "dkv_kernel"): 24.21 * GiB,
+        # the dK/dV stage at c4 is two launches: dkv_kernel (17.07 GiB) and depth_cols_kernel (7.04 GiB)
+        ("c4", "fwd_kernel"): 5.73 * GiB, ("c4", "dq_kernel"): 6.09 * GiB, ("c4", "dkv_kernel"): 24.11 * GiB,
         ("c3", "fwd_kernel"): 1.05 * GiB, ("c3", "dq_kernel"): 1.14 * GiB, ("c3", "dkv_kernel"): 2.79 * GiB,
     }
     roofline = {
