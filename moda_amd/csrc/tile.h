@@ -289,44 +289,6 @@ inline hipError_t allow_dynamic_lds(LdsAttrState& state, const void* kernel, siz
   return e;
 }
 
-// Raw buffer resource over `nbytes` bytes at `base` (wave-uniform): loads past the end return zero.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t nbytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)nbytes, 0x00020000);
-}
-
-// Cooperative global -> register -> LDS staging of a ROWS x HD tile by NT threads.
-// Global side: buffer loads with hardware range checking (rows past the end of
-// the source read as zero, no branches) and all per-pass address increments in
-// the scalar offset.  LDS side: swizzled 16-byte stores at a per-thread base
-// plus compile-time offsets.
-template <int HD, int ROWS, int NT>
-struct TileLoader {
-  static constexpr int CH = HD / 8;            // 16-byte chunks per row
-  static constexpr int RPP = NT / CH;          // rows covered per pass
-  static constexpr int N = ROWS / RPP;         // passes = 16-byte chunks per thread
-  static_assert(NT % CH == 0 && ROWS % RPP == 0 && RPP % 16 == 0, "tile must divide evenly");
-  i32x4 r[N];
-  int lds_off;  // element offset of this thread's chunk in pass 0
-
-  __device__ __forceinline__ void init(int tid) { lds_off = Tile<HD>::off(tid / CH, tid % CH); }
-
-  // src: row 0 of the (batch, head) slice; rows [row0, row0 + ROWS) are fetched, rows >= row_end read as zero.
-  __device__ __forceinline__ void load(const uint16_t* src, int64_t row_stride, int row0, int row_end, int tid) {
-    const int rows_left = row_end - row0;
-    const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
-    const uint32_t nbytes = rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
-    const __amdgpu_buffer_rsrc_t rs = make_rsrc(src + (int64_t)row0 * row_stride, nbytes);
-    const int voff = (tid / CH) * (int)stride_bytes + (tid % CH) * 16;
-#pragma unroll
-    for (int i = 0; i < N; i++)
-      r[i] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, i * RPP * (int)stride_bytes, 0));
-  }
-  __device__ __forceinline__ void store(lds_ptr tile) const {
-#pragma unroll
-    for (int i = 0; i < N; i++) *reinterpret_cast<MODA_LDS i32x4*>(tile + lds_off + i * RPP * HD) = r[i];
-  }
-};
-
 // One wave-wide direct global -> LDS load: lane l's BYTES bytes (16 or 4) land at lds_byte_addr +
 // l * BYTES; the global side is a raw buffer (descriptor rsrc, per-lane byte offset voff, scalar
 // byte offset soff) whose range check zero-fills lanes past the end.  Issued as inline assembly on
@@ -448,8 +410,6 @@ struct AsyncTileLoader {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
-
 // Combine a value with the one held by lane ^ 32 (the other half of the lane pair that shares a
 // row or column) using the gfx950 half-wave swap: {r0, r1} = {x[lane], x[lane ^ 32]} in every lane.
 __device__ __forceinline__ float pair_max(float x) {
@@ -468,32 +428,6 @@ __device__ __forceinline__ float pair_sum(float x) {
   return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
 #else
   return x;  // host pass of the single-source compile: never executed
-#endif
-}
-
-// acc + (sum of the two 16-bit values packed in w), fp32 accumulation: one instruction per pair.
-template <typename T>
-__device__ __forceinline__ float add_pair(int w, float acc);
-template <>
-__device__ __forceinline__ float add_pair<BF16>(int w, float acc) {
-  bf16x2 ones;
-  ones[0] = (__bf16)1.0f;
-  ones[1] = (__bf16)1.0f;
-#if defined(__HIP_DEVICE_COMPILE__)
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, acc, false);
-#else
-  return acc;  // host pass of the single-source compile: never executed
-#endif
-}
-template <>
-__device__ __forceinline__ float add_pair<FP16>(int w, float acc) {
-  f16x2 ones;
-  ones[0] = (_Float16)1.0f;
-  ones[1] = (_Float16)1.0f;
-#if defined(__HIP_DEVICE_COMPILE__)
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, acc, false);
-#else
-  return acc;  // host pass of the single-source compile: never executed
 #endif
 }
 
