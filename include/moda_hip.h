@@ -8,7 +8,11 @@
  * 16-byte aligned (base pointer and all strides multiples of 8 elements for
  * 16-bit types, 4 for fp32).  All work is enqueued on the hipStream_t passed
  * as `stream` (NULL = the legacy default stream); nothing synchronises the
- * host.  The library keeps no mutable state except where a function says so.
+ * host.  The library keeps no mutable state except where a function says so,
+ * apart from one flag per kernel variant and device: the first launch of a
+ * variant raises that kernel's dynamic-LDS limit (hipFuncSetAttribute), which is
+ * not a stream operation -- under stream capture (HIP graphs) make one ordinary
+ * call with the same descriptor first, then capture.
  * Every function returns 0 on success or a negative MODA_HIP_E* code; no
  * function throws.
  *
