@@ -65,7 +65,14 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   const KArgs& a = seq.a;
   const bool dep = ct >= n_seq_tiles;
   const int ncols = dep ? a.T * a.L : a.T;
-  const int c_first = (dep ? ct - n_seq_tiles : ct) * BN;
+  int tile = dep ? ct - n_seq_tiles : ct;
+  if (VARLEN && !dep && a.causal) {
+    // a causal sequence tile costs what lies behind it: count the grid's tiles from the end of the sequence, so
+    // that tiles of equal cost of all sequences are dispatched together, the heaviest of the whole batch first
+    tile -= n_seq_tiles - (a.T + BN - 1) / BN;
+    if (tile < 0) return;
+  }
+  const int c_first = tile * BN;
   if (VARLEN && c_first >= ncols) return;  // a tile beyond this sequence of a variable-length batch
   const int c = c_first + kblk * 32 + n;
   const bool valid = c < ncols;

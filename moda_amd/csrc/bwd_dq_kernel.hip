@@ -64,8 +64,11 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   SeqArgs<VARLEN> seq(a_in, b);
   const KArgs& a = seq.a;
   const int nqt = (a.Tq + BM - 1) / BM;
-  const int qt = nqt - 1 - blockIdx.x / BH;  // heavy (late) tiles first
-  if (VARLEN && qt < 0) return;  // a tile beyond this sequence of a variable-length batch
+  // Heavy (late) tiles first.  In a variable-length batch the grid counts tiles from the end of the longest
+  // sequence, so that tiles of equal cost (equal row position) of all sequences are dispatched together and the
+  // heaviest of the whole batch first; the positions a shorter sequence does not have are dropped.
+  const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
+  if (VARLEN && qt >= nqt) return;
   const int r = qt * BM + wave * 32 + n;
   const bool valid = r < a.Tq;
   const int t = r / a.Gf;
