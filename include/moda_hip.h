@@ -56,7 +56,7 @@
 extern "C" {
 #endif
 
-#define MODA_HIP_VERSION 103
+#define MODA_HIP_VERSION 104
 
 enum moda_hip_dtype { MODA_HIP_BF16 = 0, MODA_HIP_FP16 = 1, MODA_HIP_FP32 = 2 };
 
@@ -75,7 +75,8 @@ enum moda_hip_error {
   MODA_HIP_EALIGN = -3,      /* pointer or stride not 16-byte aligned               */
   MODA_HIP_EWORKSPACE = -4,  /* workspace too small                                 */
   MODA_HIP_ELAUNCH = -5,     /* hipGetLastError() reported a launch failure         */
-  MODA_HIP_EDEVICE = -6      /* current device is not gfx950                        */
+  MODA_HIP_EDEVICE = -6,     /* current device is not gfx950                        */
+  MODA_HIP_ESTATIC = -7      /* moda_hip_bwd_static: problem exceeds the built-in workspace */
 };
 
 typedef struct moda_hip_strides {
@@ -154,6 +155,24 @@ int moda_hip_bwd_stages(const moda_hip_desc* desc, const void* q, const void* k,
                         const void* kd, const void* vd, const void* o, const float* lse, const void* d_o,
                         void* dq, void* dk, void* dv, void* dkd, void* dvd,
                         void* workspace, size_t workspace_bytes, int stages, void* stream);
+
+/*
+ * moda_hip_bwd without a workspace argument and without any allocation.  No counterpart in the
+ * reference (whose launcher allocates its buffers with torch, moda_v14.py:1609-1652, 1715-1716); it is
+ * for callers that cannot allocate device memory: code under stream capture, serving loops and
+ * harnesses that forbid hipMalloc.  The row sums of o * do go to a workspace of
+ * MODA_HIP_STATIC_WORKSPACE_BYTES that is part of the library's device image (one copy per GPU, held
+ * until the process ends): problems with B * H * G * T fp32 values (packed batch: H * G * total_tokens)
+ * beyond that size are rejected with MODA_HIP_ESTATIC.  Same kernels and results as moda_hip_bwd.
+ * All calls on one GPU share the workspace: calls that may overlap on one GPU (different streams,
+ * different host threads) race; serialise them or use moda_hip_bwd with private workspaces.  The first
+ * call on a device looks the workspace address up (hipGetSymbolAddress, not a stream operation): under
+ * stream capture make one ordinary call first, as for the kernel attribute setup described above.
+ */
+#define MODA_HIP_STATIC_WORKSPACE_BYTES (8u << 20)
+int moda_hip_bwd_static(const moda_hip_desc* desc, const void* q, const void* k, const void* v,
+                        const void* kd, const void* vd, const void* o, const float* lse, const void* d_o,
+                        void* dq, void* dk, void* dv, void* dkd, void* dvd, void* stream);
 
 /*
  * Depth-KV reorganisation.  Replaces the caller-side

@@ -16,12 +16,15 @@ LIB_PATH = os.path.join(_HERE, "libmoda_hip.so")
 BF16, FP16, FP32 = 0, 1, 2
 CAUSAL, NONCAUSAL, CHUNK_VISIBLE, DEPTH_ONLY, PLAIN_GQA = 0, 1, 2, 3, 4
 STAGE_DELTA, STAGE_DQ, STAGE_DKV, STAGE_ALL = 1, 2, 4, 7
+ESTATIC = -7
+STATIC_WORKSPACE_BYTES = 8 << 20  # MODA_HIP_STATIC_WORKSPACE_BYTES
 
 EXPORTS = (
     "moda_hip_fwd",
     "moda_hip_bwd_workspace_bytes",
     "moda_hip_bwd",
     "moda_hip_bwd_stages",
+    "moda_hip_bwd_static",
     "moda_hip_depth_reorg_fwd",
     "moda_hip_depth_reorg_bwd",
     "moda_hip_strerror",
@@ -94,6 +97,8 @@ def load():
     lib.moda_hip_bwd.argtypes = [POINTER(Desc)] + [vp] * 14 + [c_size_t, vp]
     lib.moda_hip_bwd_stages.restype = c_int
     lib.moda_hip_bwd_stages.argtypes = [POINTER(Desc)] + [vp] * 14 + [c_size_t, c_int, vp]
+    lib.moda_hip_bwd_static.restype = c_int
+    lib.moda_hip_bwd_static.argtypes = [POINTER(Desc)] + [vp] * 13 + [vp]
     lib.moda_hip_depth_reorg_fwd.restype = c_int
     lib.moda_hip_depth_reorg_fwd.argtypes = [POINTER(vp), c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                              c_int64, c_int32, vp, vp]

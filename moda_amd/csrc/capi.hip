@@ -114,6 +114,25 @@ int check_device(int* compute_units = nullptr) {
   return st == 1 ? MODA_HIP_OK : MODA_HIP_EDEVICE;
 }
 
+// Workspace of moda_hip_bwd_static: lives in the code object, one copy per device the library is loaded on, for as
+// long as the process runs.  In host code the array's name is only a handle for hipGetSymbolAddress; the
+// device address is looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[MODA_HIP_STATIC_WORKSPACE_BYTES];
+
+int static_workspace(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return MODA_HIP_EDEVICE;
+  static std::atomic<void*> table[64];
+  if (dev < 0 || dev >= 64) return MODA_HIP_EDEVICE;
+  void* p = table[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MODA_HIP_ELAUNCH;
+    table[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return MODA_HIP_OK;
+}
+
 #define MODA_REQ_PTR(p) \
   if (!(p)) return MODA_HIP_EINVAL
 #define MODA_REQ_ALIGN(p, s)                              \
@@ -179,6 +198,19 @@ int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const voi
                  void* dkd, void* dvd, void* workspace, size_t workspace_bytes, void* stream) {
   return moda_hip_bwd_stages(d, q, k, v, kd, vd, o, lse, d_o, dq, dk, dv, dkd, dvd, workspace, workspace_bytes,
                              MODA_HIP_STAGE_ALL, stream);
+}
+
+int moda_hip_bwd_static(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
+                        const void* vd, const void* o, const float* lse, const void* d_o, void* dq, void* dk,
+                        void* dv, void* dkd, void* dvd, void* stream) {
+  const size_t need = moda_hip_bwd_workspace_bytes(d);
+  if (need == 0) return MODA_HIP_EINVAL;
+  if (need > (size_t)MODA_HIP_STATIC_WORKSPACE_BYTES) return MODA_HIP_ESTATIC;
+  void* ws = nullptr;
+  const int rc = static_workspace(&ws);
+  if (rc) return rc;
+  return moda_hip_bwd_stages(d, q, k, v, kd, vd, o, lse, d_o, dq, dk, dv, dkd, dvd, ws,
+                             (size_t)MODA_HIP_STATIC_WORKSPACE_BYTES, MODA_HIP_STAGE_ALL, stream);
 }
 
 int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
@@ -315,6 +347,7 @@ const char* moda_hip_strerror(int code) {
     case MODA_HIP_EWORKSPACE: return "workspace missing or too small";
     case MODA_HIP_ELAUNCH: return "HIP kernel launch failed";
     case MODA_HIP_EDEVICE: return "current device is not an MI355X-class (gfx950) GPU";
+    case MODA_HIP_ESTATIC: return "problem needs more than the MODA_HIP_STATIC_WORKSPACE_BYTES of moda_hip_bwd_static";
     default: return "unknown error";
   }
 }

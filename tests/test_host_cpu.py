@@ -32,7 +32,7 @@ def test_descriptor_layout_and_version():
     from moda_amd import _lib
 
     lib = _lib.load()
-    assert lib.moda_hip_version() == 103
+    assert lib.moda_hip_version() == 104
     assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24 + 24
     assert _lib.Desc.cu_seqlens.offset == 80 + 12 * 24
     assert _lib.Desc.q.offset == 80
