@@ -1,12 +1,16 @@
 """Headline benchmark: parallel_moda forward+backward TFLOP/s on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c2|c5|plain]
-                    [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c2|c5|c5fda|c4packed|plain]
+                    [--no-cpu-baseline] [--no-configs] [--with-stack]
+    python bench.py --summarise-pmc FETCH_DIR WRITE_DIR --workload NAME   (no GPU: rewrites profiles/hbm_traffic.json
+                    from two rocprofv3 --pmc runs of this file)
 
 A step is one forward plus one backward of the fused sequence+depth attention on
 one batch of synthetic, HBM-resident input.  The default workload is the
 long-context headline: causal, bf16, B=1, T=65536, Hq=16 (Hkv=4, G=4), D=128,
-L=24.  Prints ONE JSON line.  Only the ``cpu_baseline`` leg imports ``oracle``.
+L=24; the same line carries, under ``configs``, every other benchmark configuration (c2, c3 with their plain
+causal twins of the same shape, c5 and its depth-only variant).  Prints ONE JSON line.  Only the
+``cpu_baseline`` leg imports ``oracle``.
 """
 import argparse
 import json
@@ -30,6 +34,8 @@ WORKLOADS = {
     "c5": (64, 197, 6, 1, 64, 12, "noncausal", 0),
     "c5fda": (64, 197, 6, 1, 64, 12, "depth_only", 0),
     "plain": (1, 65536, 4, 4, 128, 0, "plain", 0),
+    "plain_c2": (2, 4096, 4, 4, 128, 0, "plain", 0),
+    "plain_c3": (1, 16384, 4, 4, 128, 0, "plain", 0),
     # the c4 token count as one packed variable-length batch (cu_seqlens): 1 x 16K, 2 x 8K, 4 x 4K, 8 x 2K tokens
     "c4packed": (1, 65536, 4, 4, 128, 24, "causal", 0),
 }
@@ -85,6 +91,7 @@ def cpu_baseline(B, T, Hkv, G, D, L, mode, cb, target_seconds=15.0):
 
     import oracle
 
+    # the GPU box gives one GPU's job a share of 16 host cores whatever os.cpu_count() shows there
     cores = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
     omode = "causal" if mode == "plain" else mode
@@ -246,6 +253,79 @@ def bench_stack(dev, steps=10):
             "inference_rebuilt_cache_ms": timed(lambda: infer(False))}
 
 
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+# what FETCH_SIZE / WRITE_SIZE (KiB per dispatch) read for a plain copy of known size (the depth reorganisation
+# kernel of the same runs): FETCH_SIZE counts half of the bytes read, WRITE_SIZE all bytes written
+PMC_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
+KERNEL_NAMES = ("fwd_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "depth_cols_kernel", "reorg_kernel")
+
+
+def recorded_traffic(workload):
+    """HBM bytes per launch and kernel from profiles/hbm_traffic.json (counters cannot be read from inside this
+    process: the file is rewritten by --summarise-pmc from rocprofv3 --pmc runs of this very command)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f)["workloads"].get(workload)
+    except (OSError, ValueError, KeyError):
+        return None
+
+
+def summarise_pmc(fetch_dir, write_dir, workload):
+    """Reads the counter_collection CSVs of `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
+    `bench.py --workload NAME --steps 1 --warmup 0 --no-cpu-baseline --no-configs` and stores, per kernel, the
+    FIRST dispatch's scaled byte count (the first dispatches belong to the workload itself; the plain twin, where
+    one runs, comes later with the same kernel names)."""
+    import csv
+    import glob
+
+    def first_dispatch(directory, counter):
+        out = {}
+        files = sorted(glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True))
+        if not files:
+            raise SystemExit(f"no counter_collection.csv under {directory}")
+        rows = []
+        for fn in files:
+            with open(fn) as f:
+                rows += [r for r in csv.DictReader(f) if r["Counter_Name"] == counter]
+        rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+        for r in rows:
+            for kn in KERNEL_NAMES:
+                if f"moda::{kn}" in r["Kernel_Name"] and kn not in out:
+                    out[kn] = float(r["Counter_Value"]) * 1024.0 * PMC_SCALE[counter]
+        return out
+
+    fetch, write = first_dispatch(fetch_dir, "FETCH_SIZE"), first_dispatch(write_dir, "WRITE_SIZE")
+    try:
+        with open(TRAFFIC_FILE) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        doc = {}
+    doc["note"] = ("HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), scaled by "
+                   f"{PMC_SCALE} (what the same counters read for the reorg_kernel copy of known size); written by "
+                   "`python bench.py --summarise-pmc`, read by bench.py for roofline.traffic")
+    doc.setdefault("workloads", {})[workload] = {
+        kn: {"fetch_bytes": fetch.get(kn, 0.0), "write_bytes": write.get(kn, 0.0),
+             "bytes": fetch.get(kn, 0.0) + write.get(kn, 0.0)}
+        for kn in KERNEL_NAMES if kn in fetch or kn in write}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(doc, f, indent=1, sort_keys=True)
+        f.write("\n")
+    for kn, v in doc["workloads"][workload].items():
+        print(f"{workload:8s} {kn:20s} read {v['fetch_bytes'] / 2**30:8.3f} GiB  written {v['write_bytes'] / 2**30:8.3f} GiB")
+
+
+def min_hbm_bytes(B, T, Hkv, G, D, L, mode):
+    """Every input read once and every output written once, forward + backward (bf16 tensors, fp32 statistics)."""
+    es = 2
+    n_q = B * T * G * Hkv * D * es
+    n_kv = 0 if mode == "depth_only" else B * T * Hkv * D * es
+    n_dep = B * T * L * Hkv * D * es
+    n_stat = B * T * G * Hkv * 4
+    fwd = n_q + 2 * n_kv + 2 * n_dep + n_q + n_stat
+    bwd = 2 * n_q + 2 * n_kv + 2 * n_dep + n_q + 2 * n_stat + n_q + 2 * n_kv + 2 * n_dep + 2 * n_stat
+    return fwd + bwd
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -253,10 +333,17 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the `configs` object (the other benchmark configurations and their plain twins)")
     ap.add_argument("--with-twin", action="store_true", help="also time the plain causal twin (c4 shape, no depth)")
     ap.add_argument("--with-stack", action="store_true",
                     help="also time a 12-block attention+MLP stack chained through the depth stream")
+    ap.add_argument("--summarise-pmc", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="no GPU work: rewrite profiles/hbm_traffic.json for --workload from two rocprofv3 --pmc runs")
     args = ap.parse_args()
+    if args.summarise_pmc:
+        summarise_pmc(args.summarise_pmc[0], args.summarise_pmc[1], args.workload)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards over batch and kv heads without exchange "
               "but no multi-GPU launch is implemented. Use --gpus 1.", file=sys.stderr)
@@ -334,6 +421,19 @@ def main():
         return {"ms_step": ms_step, "flops_fwd": ff, "t_fwd": t_fwd, "t_delta": t_delta, "t_dq": t_dq,
                 "t_dkv": t_dkv, "shape": (B, T, Hkv, G, D, L, mode, cb)}
 
+    def describe(name, shape):
+        B, T, Hkv, G, D, L, mode, cb = shape
+        return (f"{name}: {mode} B={B} T={T} Hq={Hkv * G} Hkv={Hkv} G={G} D={D} L={L}"
+                + (f" chunk_tokens={cb}" if cb else "")
+                + (f" packed sequence lengths={PACKED_LENGTHS[name]}" if name in PACKED_LENGTHS else ""))
+
+    def hbm_bound(shape, total_flops):
+        """Small shapes (DeiT-sized c5, depth-only attention) are bound by HBM, not by the matrix pipe: reading
+        every input once and writing every output once already takes longer than their FLOPs at the MFMA peak."""
+        B, T, Hkv, G, D, L, mode, cb = shape
+        return mode != "plain" and total_flops / min_hbm_bytes(B, T, Hkv, G, D, L, mode) \
+            < PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+
     r = run_workload(args.workload, args.steps, args.warmup)
     B, T, Hkv, G, D, L, mode, cb = r["shape"]
     total_flops = 3.5 * r["flops_fwd"]
@@ -350,43 +450,32 @@ def main():
         "dkv_kernel": {"ms": r["t_dkv"], "tflops": 3 * unit / (r["t_dkv"] * 1e-3) / 1e12},
     }
     dom = max(("fwd_kernel", "dq_kernel", "dkv_kernel"), key=lambda n: kernels[n]["ms"])
-    # HBM bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file (one counter per
-    # run), FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 (what the same counters read for the depth
-    # reorganisation copy of known size).  Counters cannot be read from inside this process, so the
-    # figures are recorded here per workload and kernel; a workload without a recorded run reports null.
-    GiB = float(1 << 30)
-    measured_hbm_bytes = {
-        # the dK/dV stage at c4 is two launches: dkv_kernel (17.07 GiB) and depth_cols_kernel (7.04 GiB)
-        ("c4", "fwd_kernel"): 5.73 * GiB, ("c4", "dq_kernel"): 6.09 * GiB, ("c4", "dkv_kernel"): 24.11 * GiB,
-        ("c3", "fwd_kernel"): 1.05 * GiB, ("c3", "dq_kernel"): 1.14 * GiB, ("c3", "dkv_kernel"): 2.79 * GiB,
-    }
+    traffic = recorded_traffic(args.workload) or {}
+    # the dK/dV stage is timed as a whole: outside chunk-visible mode it is dkv_kernel followed by the HBM-bound
+    # depth_cols_kernel
+    two_launches = dom == "dkv_kernel" and L > 0 and mode != "chunk_visible"
+    dom_traffic = None
+    if dom in traffic:
+        dom_traffic = traffic[dom]["bytes"] + (traffic.get("depth_cols_kernel", {}).get("bytes", 0.0) if two_launches else 0.0)
     roofline = {
         "bound": "mfma",
-        # the dK/dV stage is timed as a whole: outside chunk-visible mode it is dkv_kernel followed by the
-        # HBM-bound depth_cols_kernel (5 % of the stage at c4)
-        "kernel": "dkv_kernel + depth_cols_kernel" if (dom == "dkv_kernel" and L > 0 and mode != "chunk_visible") else dom,
+        "kernel": "dkv_kernel + depth_cols_kernel" if two_launches else dom,
         "achieved": kernels[dom]["tflops"],
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS,
-        "traffic": measured_hbm_bytes.get((args.workload, dom)),
+        "traffic": dom_traffic,
+        "traffic_source": "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
+                          "recorded, not measured by this run)" if dom_traffic is not None else None,
     }
-    # Small shapes (DeiT-sized c5, depth-only attention) are bound by HBM, not by the matrix pipe: every input
-    # read once and every output written once already takes longer than their FLOPs at the MFMA peak.  For
-    # those the roofline object is the whole step against the HBM peak.
-    es = 2
-    Tq, Hq_rows = T * G, Hkv
-    n_q = B * Tq * Hq_rows * D * es
-    n_kv = (0 if mode == "depth_only" else B * T * Hkv * D * es)
-    n_dep = B * T * L * Hkv * D * es
-    n_stat = B * Tq * Hq_rows * 4
-    min_bytes = (n_q + 2 * n_kv + 2 * n_dep + n_q + n_stat) \
-        + (2 * n_q + 2 * n_kv + 2 * n_dep + n_q + 2 * n_stat + n_q + 2 * n_kv + 2 * n_dep + 2 * n_stat)
-    if mode != "plain" and total_flops / min_bytes < PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9):
-        gbs = min_bytes / (r["ms_step"] * 1e-3) / 1e9
+    if hbm_bound(r["shape"], total_flops):
+        mb = min_hbm_bytes(B, T, Hkv, G, D, L, mode)
+        gbs = mb / (r["ms_step"] * 1e-3) / 1e9
+        whole = sum(v["bytes"] for v in traffic.values()) if traffic else None
         roofline = {"bound": "hbm", "kernel": "fwd_kernel + delta_kernel + dq_kernel + dkv_kernel + depth_cols_kernel",
                     "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                    "algorithmic_bytes": min_bytes, "traffic": None}
+                    "algorithmic_bytes": mb, "traffic": whole,
+                    "traffic_source": "profiles/hbm_traffic.json (recorded)" if whole is not None else None}
     out = {
         "metric": "parallel_moda fwd+bwd TFLOP/s at T=64K bf16; % of bf16 MFMA peak",
         "value": value,
@@ -400,11 +489,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {mode} B={B} T={T} Hq={Hkv * G} Hkv={Hkv} G={G} D={D} L={L}"
-                               + (f" chunk_tokens={cb}" if cb else "")
-                               + (f" packed sequence lengths={PACKED_LENGTHS[args.workload]}"
-                                  if args.workload in PACKED_LENGTHS else ""),
-                   "flop_fwd_bwd": total_flops},
+        "config": {"workload": describe(args.workload, r["shape"]), "flop_fwd_bwd": total_flops},
         "frac_of_bf16_mfma_peak": value / PEAK_BF16_TFLOPS,
         "kernels": kernels,
         "roofline": roofline,
@@ -414,6 +499,32 @@ def main():
         tw_value = 3.5 * tw["flops_fwd"] / (tw["ms_step"] * 1e-3) / 1e12
         out["plain_causal_twin"] = {"tflops": tw_value, "ms_per_step": tw["ms_step"],
                                     "moda_over_twin": value / tw_value}
+    if args.workload == "c4" and not args.no_configs:
+        # every other benchmark configuration in the same run: absolute rate, fraction of the matching peak,
+        # per-kernel times, and for the matrix-bound ones the plain causal twin of the same shape
+        configs = {}
+        for name, twin in (("c2", "plain_c2"), ("c3", "plain_c3"), ("c5", None), ("c5fda", None)):
+            torch.cuda.empty_cache()
+            c = run_workload(name, 20, 5)
+            fl = 3.5 * c["flops_fwd"]
+            tf = fl / (c["ms_step"] * 1e-3) / 1e12
+            entry = {"workload": describe(name, c["shape"]), "ms": c["ms_step"], "tflops": tf,
+                     "frac_of_bf16_mfma_peak": tf / PEAK_BF16_TFLOPS, "flop_fwd_bwd": fl,
+                     "kernel_ms": {"fwd": c["t_fwd"], "delta": c["t_delta"], "dq": c["t_dq"], "dkv": c["t_dkv"]}}
+            if hbm_bound(c["shape"], fl):
+                cB, cT, cH, cG, cD, cL, cmode, _ = c["shape"]
+                mb = min_hbm_bytes(cB, cT, cH, cG, cD, cL, cmode)
+                entry.update({"bound": "hbm", "algorithmic_bytes": mb, "gbs": mb / (c["ms_step"] * 1e-3) / 1e9,
+                              "frac_of_hbm_peak": mb / (c["ms_step"] * 1e-3) / 1e9 / PEAK_HBM_GBS})
+            else:
+                entry["bound"] = "mfma"
+            if twin:
+                t = run_workload(twin, 20, 5)
+                ttf = 3.5 * t["flops_fwd"] / (t["ms_step"] * 1e-3) / 1e12
+                entry["plain_causal_twin"] = {"ms": t["ms_step"], "tflops": ttf, "moda_over_twin": tf / ttf}
+            configs[name] = entry
+        out["configs"] = configs
+        torch.cuda.empty_cache()
     if L > 0:
         out["depth_reorg"] = bench_reorg(dev, B, T, Hkv, D, L)
     probe = bench_mfma_probe(dev)

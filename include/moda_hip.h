@@ -4,9 +4,11 @@
  * cache reorganisation.
  *
  * Every pointer that names tensor data is a DEVICE pointer.  Strides are in
- * elements; the innermost (head-dim) stride is always 1 and every row must be
- * 16-byte aligned (base pointer and all strides multiples of 8 elements for
- * 16-bit types, 4 for fp32).  All work is enqueued on the hipStream_t passed
+ * elements; the innermost (head-dim) stride is always 1.  For the matrix-core
+ * kernels (bf16/fp16, head dim 64 or 128, Dv == D) every row must be 16-byte
+ * aligned (base pointer and all strides multiples of 8 elements) and a row
+ * stride must stay below 16 MiB; every other combination runs on vector-ALU
+ * kernels that need element alignment only.  All work is enqueued on the hipStream_t passed
  * as `stream` (NULL = the legacy default stream); nothing synchronises the
  * host.  The library keeps no mutable state except where a function says so,
  * apart from one flag per kernel variant and device: the first launch of a
@@ -79,6 +81,19 @@ enum moda_hip_error {
   MODA_HIP_ESTATIC = -7      /* moda_hip_bwd_static: problem exceeds the built-in workspace */
 };
 
+enum moda_hip_flag {
+  /*
+   * Backward adds the depth-stream gradients to what dkd, dvd already hold (one rounding to the
+   * tensor type per call) instead of overwriting them, and leaves the slots l >= L_valid untouched.
+   * With one preallocated depth cache per model and one gradient buffer of the same shape, the
+   * backward of layer n (L_valid = n) then adds its share to slots < n, and a layer's K/V gradient is
+   * a slice of that buffer: no per-layer rebuild of the cache and no scatter of its gradient
+   * (vision_tasks/deit/models.py:361-390 does both for every layer).  Still one writer per row and
+   * no atomics.  Not available with MODA_HIP_CHUNK_VISIBLE.
+   */
+  MODA_HIP_FLAG_ACCUMULATE_DEPTH_GRADS = 1
+};
+
 typedef struct moda_hip_strides {
   int64_t b; /* batch stride   */
   int64_t t; /* row stride     */
@@ -98,7 +113,7 @@ typedef struct moda_hip_desc {
   int64_t L;            /* depth slots per token, 0 = no depth stream              */
   int64_t chunk_tokens; /* CHUNK_VISIBLE: base tokens per chunk (C / G), else 0    */
   float scale;          /* logits = scale * <q, key>                               */
-  float reserved_f;
+  int32_t flags;        /* OR of moda_hip_flag values, 0 = none                    */
   moda_hip_strides q, k, v, kd, vd, o, d_o, dq, dk, dv, dkd, dvd;
   const int32_t* cu_seqlens; /* packed variable-length batch (see above): DEVICE array of B + 1 offsets, else NULL */
   int64_t total_tokens;      /* with cu_seqlens: cu_seqlens[B], the length of the packed token axis              */

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libmoda_hip.so")
 BF16, FP16, FP32 = 0, 1, 2
 CAUSAL, NONCAUSAL, CHUNK_VISIBLE, DEPTH_ONLY, PLAIN_GQA = 0, 1, 2, 3, 4
 STAGE_DELTA, STAGE_DQ, STAGE_DKV, STAGE_ALL = 1, 2, 4, 7
+FLAG_ACCUMULATE_DEPTH_GRADS = 1
 ESTATIC = -7
 STATIC_WORKSPACE_BYTES = 8 << 20  # MODA_HIP_STATIC_WORKSPACE_BYTES
 
@@ -51,7 +52,7 @@ class Desc(Structure):
         ("L", c_int64),
         ("chunk_tokens", c_int64),
         ("scale", c_float),
-        ("reserved_f", c_float),
+        ("flags", c_int32),
         ("q", Strides),
         ("k", Strides),
         ("v", Strides),

@@ -406,7 +406,8 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   const int w = (int)(c / a.L), slot = (int)(c - (int64_t)w * a.L);
   uint16_t* dk_out = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + c * a.sdkd.t + 8 * sub;
   uint16_t* dv_out = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + c * a.sdvd.t + 8 * sub;
-  if (slot >= a.Lv) {  // a slot without data
+  if (slot >= a.Lv) {  // a slot without data: zero gradient, or (accumulating) somebody else's sum to leave alone
+    if (a.accum_depth) return;
     const i32x4 z = {0, 0, 0, 0};
     *reinterpret_cast<i32x4*>(dk_out) = z;
     *reinterpret_cast<i32x4*>(dv_out) = z;
@@ -452,10 +453,22 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
       dk[i] = __builtin_fmaf(ds, qf[i], dk[i]);
     }
   }
+#pragma unroll
+  for (int i = 0; i < 8; i++) dk[i] *= a.scale;
+  if (a.accum_depth) {  // add to what the row holds (this thread is its only writer), one rounding per call
+    float ok_old[8], ov_old[8];
+    load8(dk_out, ok_old);
+    load8(dv_out, ov_old);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      dk[i] += ok_old[i];
+      dv[i] += ov_old[i];
+    }
+  }
   i32x4 ok, ov;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    ok[i] = pack2<T>(dk[2 * i] * a.scale, dk[2 * i + 1] * a.scale);
+    ok[i] = pack2<T>(dk[2 * i], dk[2 * i + 1]);
     ov[i] = pack2<T>(dv[2 * i], dv[2 * i + 1]);
   }
   *reinterpret_cast<i32x4*>(dk_out) = ok;

@@ -2,7 +2,8 @@
 // dQ kernel (moda_v14.py:542-871, moda_v16.py:936-1220, fda_v12.py:432-638,
 // fla/ops/attn/parallel.py:165-296).
 //
-// Same decomposition as the forward kernel: a workgroup owns 128 query rows,
+// Same decomposition as the forward kernel: a workgroup owns 32 query rows per wave
+// (256 in the throughput launch shape, 64 or 128 in the small one),
 // one row per lane pair, and streams 64-column K/V tiles (sequence keys, then
 // the rows' depth slots).  P^T is recomputed from the saved base-2 LSE,
 // dS^T = P^T * (dP^T - delta) is packed straight into the B operand of

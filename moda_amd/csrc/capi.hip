@@ -29,7 +29,10 @@ int elem_size(int dtype) { return dtype == MODA_HIP_FP32 ? 4 : 2; }
 
 Str3 cvt(const moda_hip_strides& s) { return Str3{s.b, s.t, s.h}; }
 
-bool aligned(const void* p, const moda_hip_strides& s, int esize) {
+// The MFMA kernels move rows with 16-byte accesses; the vector-ALU kernels load element by element and
+// need element alignment only.
+bool aligned(const void* p, const moda_hip_strides& s, int esize, bool vec16) {
+  if (!vec16) return (uintptr_t)p % esize == 0;
   const int64_t m = 16 / esize;
   return ((uintptr_t)p % 16 == 0) && (s.b % m == 0) && (s.t % m == 0) && (s.h % m == 0);
 }
@@ -59,6 +62,8 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L > 0 && d->chunk_tokens <= 0) return MODA_HIP_EINVAL;
   if (d->L_valid < 0 || d->L_valid > d->L) return MODA_HIP_EINVAL;
   if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L_valid != 0 && d->L_valid != d->L) return MODA_HIP_EUNSUPPORTED;
+  if (d->flags & ~(int32_t)MODA_HIP_FLAG_ACCUMULATE_DEPTH_GRADS) return MODA_HIP_EINVAL;
+  if ((d->flags & MODA_HIP_FLAG_ACCUMULATE_DEPTH_GRADS) && d->mode == MODA_HIP_CHUNK_VISIBLE) return MODA_HIP_EUNSUPPORTED;
   // 32-bit index space used for rows and flattened depth columns inside the kernels
   if (d->T * d->G >= (1ll << 30) || d->T * (d->L > 0 ? d->L : 1) >= (1ll << 30) || d->B * d->H * d->G >= (1ll << 20))
     return MODA_HIP_EUNSUPPORTED;
@@ -77,6 +82,7 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   a.has_seq = d->mode != MODA_HIP_DEPTH_ONLY;
   a.causal = d->mode == MODA_HIP_CAUSAL || d->mode == MODA_HIP_CHUNK_VISIBLE || plain;
   a.chunk = d->mode == MODA_HIP_CHUNK_VISIBLE;
+  a.accum_depth = (d->flags & MODA_HIP_FLAG_ACCUMULATE_DEPTH_GRADS) ? 1 : 0;
   a.nqt = (a.Tq + 127) / 128;
   a.scale = d->scale;
   a.delta_pitch = a.Tq;
@@ -135,9 +141,9 @@ int static_workspace(void** out) {
 
 #define MODA_REQ_PTR(p) \
   if (!(p)) return MODA_HIP_EINVAL
-#define MODA_REQ_ALIGN(p, s)                              \
-  if (!aligned((p), (s), es)) return MODA_HIP_EALIGN; \
-  if (!row_stride_ok((s), es)) return MODA_HIP_EUNSUPPORTED
+#define MODA_REQ_ALIGN(p, s)                                    \
+  if (!aligned((p), (s), es, vec16)) return MODA_HIP_EALIGN; \
+  if (vec16 && !row_stride_ok((s), es)) return MODA_HIP_EUNSUPPORTED
 
 }  // namespace
 
@@ -150,6 +156,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
   if (rc) return rc;
   if ((int64_t)a.B * a.Tq * a.Hq == 0) return MODA_HIP_OK;
   const int es = elem_size(d->dtype);
+  const bool vec16 = use_mfma(d);
   MODA_REQ_PTR(q);
   MODA_REQ_PTR(o);
   MODA_REQ_PTR(lse);
@@ -222,6 +229,7 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
   if (rc) return rc;
   if (stages < 0 || stages > MODA_HIP_STAGE_ALL) return MODA_HIP_EINVAL;
   const int es = elem_size(d->dtype);
+  const bool vec16 = use_mfma(d);
   const bool have_rows = (int64_t)a.B * a.Tq * a.Hq > 0;
   if (have_rows) {
     MODA_REQ_PTR(q);

@@ -206,7 +206,10 @@ __global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, cons
     const int w = col / a.L;
     qlo = w * a.Gf;
     qhi = a.chunk ? min(a.T, (w / a.Cb + 1) * a.Cb) * a.Gf : (w + 1) * a.Gf;
-    if (col - w * a.L >= a.Lv) qhi = qlo;  // a slot without data: no row sees it, its gradients are zero
+    if (col - w * a.L >= a.Lv) {  // a slot without data: no row sees it
+      if (a.accum_depth) return;  // accumulating: the row holds somebody else's sum
+      qhi = qlo;                  // its gradients are zero
+    }
   }
   float dk[kDR], dv[kDR];
 #pragma unroll
@@ -261,8 +264,9 @@ __global__ __launch_bounds__(256) void generic_col_kernel(const KArgs a_in, cons
 #pragma unroll
   for (int i = 0; i < kDR; i++) {
     const int d = lane + 64 * i;
-    if (d < D) st<E>(dkp, dkoff + d, dk[i] * a.scale);
-    if (d < Dv) st<E>(dvp, dvoff + d, dv[i]);
+    const bool add = dep && a.accum_depth;  // this wave is the row's only writer
+    if (d < D) st<E>(dkp, dkoff + d, dk[i] * a.scale + (add ? ld<E>(dkp, dkoff + d) : 0.f));
+    if (d < Dv) st<E>(dvp, dvoff + d, dv[i] + (add ? ld<E>(dvp, dvoff + d) : 0.f));
   }
 }
 

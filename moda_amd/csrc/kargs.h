@@ -24,6 +24,7 @@ struct KArgs {
   int Lv;    // slots per token that hold data, 1 <= Lv <= L: slots l >= Lv are invisible
   int Cb;    // chunk-visible: tokens per chunk
   int has_seq, causal, chunk;
+  int accum_depth;  // dkd, dvd += (slots l >= Lv untouched) instead of = (slots l >= Lv zeroed)
   int nqt;   // query tiles per (batch, query head)
   float scale;
   int compute_units;  // of the device the launch goes to (host-side launch-shape decisions)

@@ -27,6 +27,14 @@ def _ptr_array(tensors: Sequence[torch.Tensor]):
 
 def _reorg_fwd(layers: Sequence[torch.Tensor], cache: torch.Tensor, slot0: int, L_total: int):
     B, T, H, D = layers[0].shape
+    # the C ABI sees bare pointers: every extent it will touch is checked here
+    assert tuple(cache.shape) == (B, T * L_total, H, D) and cache.is_contiguous(), \
+        f"cache must be a contiguous {(B, T * L_total, H, D)} tensor, got {tuple(cache.shape)}"
+    assert 0 <= slot0 and slot0 + len(layers) <= L_total, "slots out of range"
+    for x in layers:
+        assert tuple(x.shape) == (B, T, H, D) and x.is_contiguous(), "every layer must be a contiguous [B, T, H, D] tensor"
+        assert x.dtype == cache.dtype and x.device == cache.device, "layers and cache must share dtype and device"
+    _check_device(cache)
     with torch.cuda.device(cache.device):
         rc = _lib.load().moda_hip_depth_reorg_fwd(_ptr_array(layers), len(layers), slot0, L_total, B, T, H, D,
                                                   _DTYPES[cache.dtype], ctypes.c_void_p(cache.data_ptr()),
@@ -36,6 +44,10 @@ def _reorg_fwd(layers: Sequence[torch.Tensor], cache: torch.Tensor, slot0: int, 
 
 def _reorg_bwd(d_cache: torch.Tensor, n_layers: int, slot0: int, L_total: int, shape) -> List[torch.Tensor]:
     B, T, H, D = shape
+    assert tuple(d_cache.shape) == (B, T * L_total, H, D) and d_cache.is_contiguous(), \
+        f"d_cache must be a contiguous {(B, T * L_total, H, D)} tensor, got {tuple(d_cache.shape)}"
+    assert 0 <= slot0 and slot0 + n_layers <= L_total, "slots out of range"
+    _check_device(d_cache)
     outs = [torch.empty(B, T, H, D, dtype=d_cache.dtype, device=d_cache.device) for _ in range(n_layers)]
     with torch.cuda.device(d_cache.device):
         rc = _lib.load().moda_hip_depth_reorg_bwd(ctypes.c_void_p(d_cache.data_ptr()), n_layers, slot0, L_total, B, T,
@@ -95,6 +107,10 @@ class DepthCache:
 
     def append(self, k: torch.Tensor, v: torch.Tensor):
         assert self.n < self.L_max, "depth cache is full"
+        for name, x in (("k", k), ("v", v)):
+            assert tuple(x.shape) == self.shape, f"{name} must be {self.shape} like the cache, got {tuple(x.shape)}"
+            assert x.dtype == self.k.dtype and x.device == self.k.device, \
+                f"{name} must have the cache's dtype ({self.k.dtype}) and device"
         _reorg_fwd([k.contiguous()], self.k, self.n, self.L_max)
         _reorg_fwd([v.contiguous()], self.v, self.n, self.L_max)
         self.n += 1

@@ -71,12 +71,16 @@ def _stream(x: torch.Tensor):
     return ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
 
 
-def _usable(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+def _usable(x: Optional[torch.Tensor], vec16: bool = True) -> Optional[torch.Tensor]:
     """Return ``x`` if the kernels can read it in place (unit inner stride, 16-byte
     aligned rows), else a contiguous copy -- the reference's ``@contiguous``
-    (fla/utils.py:130-164) made a copy of every non-contiguous input."""
+    (fla/utils.py:130-164) made a copy of every non-contiguous input.  ``vec16=False``: the
+    vector-ALU kernels, which load element by element and take any non-negative strides."""
     if x is None:
         return None
+    if not vec16:
+        ok = x.dim() == 4 and (x.stride(3) == 1 or x.shape[3] == 1) and all(x.stride(i) >= 0 for i in range(3))
+        return x if ok else x.contiguous()
     m = 16 // x.element_size()
     ok = (
         x.dim() == 4
@@ -87,6 +91,11 @@ def _usable(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
         and x.stride(1) * x.element_size() < (1 << 24)  # row offsets inside a tile are 32-bit
     )
     return x if ok else x.contiguous()
+
+
+def _matrix_core_path(q: torch.Tensor, val: torch.Tensor) -> bool:
+    """Whether the call runs on the matrix-core kernels (16-bit, head dim 64 or 128 for keys and values)."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[3] in (64, 128) and val.shape[3] == q.shape[3]
 
 
 def _strides(x: Optional[torch.Tensor]) -> Strides:
@@ -103,7 +112,7 @@ def _check_device(x: torch.Tensor):
 
 
 def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=None, dk=None, dv=None, dkd=None,
-          dvd=None, depth_valid=None, packed: Optional[PackedBatch] = None) -> Desc:
+          dvd=None, depth_valid=None, packed: Optional[PackedBatch] = None, accumulate_depth=False) -> Desc:
     d = Desc()
     d.struct_size = ctypes.sizeof(Desc)
     if q.dtype not in _DTYPES:
@@ -130,6 +139,7 @@ def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=
         d.cu_seqlens = packed.cu.data_ptr()
         d.total_tokens = packed.total
     d.chunk_tokens = chunk_tokens
+    d.flags = _lib.FLAG_ACCUMULATE_DEPTH_GRADS if accumulate_depth else 0
     d.scale = float(scale)
     d.q, d.k, d.v, d.kd, d.vd = _strides(q), _strides(k), _strides(v), _strides(kd), _strides(vd)
     d.o, d.d_o = _strides(o), _strides(do)
@@ -148,11 +158,62 @@ def _same_dtype(*xs):
             raise TypeError(f"all tensors must share one dtype, got {dt} and {x.dtype}")
 
 
+def _check_shapes(mode, q, k, v, kd, vd, G, o=None, do=None, lse=None):
+    """The C ABI takes bare pointers: it derives every extent from ``k`` (or ``q``), ``G`` and the depth
+    row count and cannot see what the buffers really hold.  A mismatch would be an out-of-bounds access
+    on the device, so every extent is checked here, before any launch.  Returns ``(T, L)``."""
+    assert q.dim() == 4, "q must be [B, rows, heads, D]"
+    B = q.shape[0]
+    assert G >= 1, "moda_group_num must be positive"
+    if mode == _lib.DEPTH_ONLY:
+        assert k is None and v is None, "depth-only attention takes no sequence k/v"
+        assert kd is not None and vd is not None, "depth-only attention needs the depth k/v"
+        assert q.shape[1] % G == 0, "query rows must be a multiple of moda_group_num"
+        T, H = q.shape[1] // G, kd.shape[2]
+        assert q.shape[2] == H, "q and depth k/v must have the same number of heads"
+    else:
+        assert k is not None and v is not None and k.dim() == 4 and v.dim() == 4, "k, v must be [B, T, H, D]"
+        T, H = k.shape[1], k.shape[2]
+        assert k.shape[0] == B and v.shape[0] == B, "batch sizes of q, k, v differ"
+        assert v.shape[1] == T and v.shape[2] == H, "k and v must agree in tokens and heads"
+        assert k.shape[3] == q.shape[3], "q and k must share the head dim"
+        if mode == _lib.PLAIN_GQA:
+            assert q.shape[1] == T and q.shape[2] == H * G, "plain GQA: q must be [B, T, H*G, D]"
+        else:
+            assert q.shape[2] == H, "folded layout: q and k must have the same number of heads"
+            assert q.shape[1] == T * G, f"q holds {q.shape[1]} rows, expected T*moda_group_num = {T * G}"
+    L = 0
+    if kd is not None or vd is not None:
+        assert kd is not None and vd is not None, "depth k and v must be given together"
+        assert kd.dim() == 4 and vd.dim() == 4, "depth k/v must be [B, T*L, H, D]"
+        assert kd.shape[0] == B and vd.shape[0] == B, "depth k/v batch size differs from q"
+        assert kd.shape[2] == H and vd.shape[2] == H, "depth k/v head count mismatch"
+        assert kd.shape[3] == q.shape[3], "depth k must share q's head dim"
+        assert vd.shape[1] == kd.shape[1], "depth k and v must have the same number of rows"
+        if T > 0:
+            assert kd.shape[1] % T == 0, "depth rows must be T * L"
+            L = kd.shape[1] // T
+        else:
+            assert kd.shape[1] == 0, "depth rows must be T * L"
+        if v is not None:
+            assert vd.shape[3] == v.shape[3], "v and depth v must share the value head dim"
+    Dv = (vd if mode == _lib.DEPTH_ONLY else v).shape[3]
+    for name, x in (("o", o), ("do", do)):
+        if x is not None:
+            assert tuple(x.shape) == (B, q.shape[1], q.shape[2], Dv), f"{name} must be {(B, q.shape[1], q.shape[2], Dv)}"
+    if lse is not None:
+        assert tuple(lse.shape) == (B, q.shape[1], q.shape[2]) and lse.dtype == torch.float32, \
+            "lse must be fp32 [B, rows, heads]"
+    return T, L
+
+
 def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None, packed=None):
     """Launch the forward kernels. Returns (o, lse)."""
+    _check_shapes(mode, q, k, v, kd, vd, G)
     _check_device(q)
     _same_dtype(q, k, v, kd, vd)
-    q, k, v, kd, vd = map(_usable, (q, k, v, kd, vd))
+    vec16 = _matrix_core_path(q, vd if mode == _lib.DEPTH_ONLY else v)
+    q, k, v, kd, vd = (_usable(x, vec16) for x in (q, k, v, kd, vd))
     src = kd if mode == _lib.DEPTH_ONLY else k
     T = q.shape[1] // G if mode == _lib.DEPTH_ONLY else k.shape[1]
     L = (kd.shape[1] // T) if (kd is not None and T > 0) else 0
@@ -172,19 +233,28 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None, 
 
 
 def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages=_lib.STAGE_ALL, out=None, ws=None,
-             depth_valid=None, packed=None):
+             depth_valid=None, packed=None, accumulate_depth=False):
     """Launch the backward kernels. Returns (dq, dk, dv, dkd, dvd).
 
     ``stages`` selects a subset of {delta, dq, dk/dv}; ``out`` (a previous return
-    value) and ``ws`` (a workspace tensor) let the caller reuse buffers across calls."""
+    value) and ``ws`` (a workspace tensor) let the caller reuse buffers across calls.
+    ``accumulate_depth``: the depth gradients are ADDED to the ``dkd, dvd`` given in ``out`` (slots
+    ``>= depth_valid`` untouched) instead of overwriting them."""
+    assert not accumulate_depth or (out is not None and out[3] is not None and out[4] is not None), \
+        "accumulate_depth needs the gradient buffers to add to"
+    _check_shapes(mode, q, k, v, kd, vd, G, o=o, do=do, lse=lse)
     _check_device(q)
     _same_dtype(q, k, v, kd, vd, o, do)
-    q, k, v, kd, vd, o, do = map(_usable, (q, k, v, kd, vd, o, do))
+    vec16 = _matrix_core_path(q, vd if mode == _lib.DEPTH_ONLY else v)
+    q, k, v, kd, vd, o, do = (_usable(x, vec16) for x in (q, k, v, kd, vd, o, do))
     lse = lse.contiguous()
     T = q.shape[1] // G if mode == _lib.DEPTH_ONLY else k.shape[1]
     L = (kd.shape[1] // T) if (kd is not None and T > 0) else 0
     if out is not None:
         dq, dk, dv, dkd, dvd = out
+        for g_, x_ in ((dq, q), (dk, k), (dv, v), (dkd, kd), (dvd, vd)):
+            assert (g_ is None) == (x_ is None) and (g_ is None or (g_.shape == x_.shape and g_.dtype == x_.dtype)), \
+                "reused gradient buffers must match their inputs in shape and dtype"
     else:
         dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         dk = torch.empty(k.shape, dtype=k.dtype, device=q.device) if k is not None else None
@@ -193,7 +263,7 @@ def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages
         dvd = torch.empty(vd.shape, dtype=vd.dtype, device=q.device) if vd is not None else None
     kd_a, vd_a, dkd_a, dvd_a = (kd, vd, dkd, dvd) if L > 0 else (None, None, None, None)
     d = _desc(mode, q, k, v, kd_a, vd_a, G, L, chunk_tokens, scale, o=o, do=do, dq=dq, dk=dk, dv=dv, dkd=dkd_a,
-              dvd=dvd_a, depth_valid=depth_valid, packed=packed)
+              dvd=dvd_a, depth_valid=depth_valid, packed=packed, accumulate_depth=accumulate_depth and L > 0)
     lib = _lib.load()
     nbytes = lib.moda_hip_bwd_workspace_bytes(ctypes.byref(d))
     if ws is None:
@@ -365,7 +435,10 @@ def parallel_moda(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_
     ignored.  ``depth_valid`` (an extension): ``cached_k/v`` keep ``L`` slots per token
     but only the first ``depth_valid`` are visible -- the result equals that for the
     compacted ``[B, T*depth_valid, H, D]`` tensors, the gradients of the other slots are
-    zero, and a preallocated cache (``DepthCache``) need not be rebuilt per layer.
+    zero, and a preallocated cache (``DepthCache``) need not be rebuilt per layer.  The kernels still
+    read the other slots and multiply them by zero: they must hold FINITE values (``DepthCache`` and
+    ``DepthStream`` start their buffers as zeros; a ``torch.empty`` buffer may hold NaN/Inf bit patterns
+    that would turn the outputs into NaN).
     """
     q, k, v, g, cached_k, cached_v, scale = _prepare_inputs(
         "parallel_moda", q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first, return_depth_grads,

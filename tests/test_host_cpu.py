@@ -157,6 +157,68 @@ def test_argument_contract_matches_reference():
             moda_amd.parallel_moda(z(1, 2, 4, 64), z(1, 2, 4, 64), z(1, 2, 4, 64))
 
 
+def test_low_level_entry_points_check_every_extent_before_launching():
+    """The C ABI takes bare pointers and derives all extents from k, G and the depth row count; a tensor that
+    does not match would be read or written out of bounds on the device.  The host refuses such calls before
+    anything is launched (these run on CPU tensors: the shape check comes before the device check)."""
+    import moda_amd
+    from moda_amd import _lib, ops
+
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16)
+    q, k, v = z(1, 16, 2, 64), z(1, 8, 2, 64), z(1, 8, 2, 64)
+    kd, vd = z(1, 24, 2, 64), z(1, 24, 2, 64)
+    lse, o, do = torch.zeros(1, 16, 2), z(1, 16, 2, 64), z(1, 16, 2, 64)
+    # a wrong moda_group_num: q rows != T * G
+    with pytest.raises(AssertionError, match="expected T\\*moda_group_num"):
+        moda_amd.parallel_moda_fwd(q, k, v, None, 0.125, cached_k=kd, cached_v=vd, moda_group_num=1)
+    with pytest.raises(AssertionError, match="expected T\\*moda_group_num"):
+        moda_amd.parallel_moda_bwd(q, k, v, o, None, lse, do, 0.125, cached_k=kd, cached_v=vd, moda_group_num=4)
+    with pytest.raises(AssertionError, match="expected T\\*moda_group_num"):
+        moda_amd.parallel_moda_chunk_visible_fwd(q, k, v, None, 0.125, cached_k=kd, cached_v=vd, moda_group_num=1)
+    # depth rows that are not T * L, depth v shorter than depth k
+    with pytest.raises(AssertionError, match="depth rows must be T \\* L"):
+        moda_amd.parallel_moda_fwd(q, k, v, None, 0.125, cached_k=z(1, 20, 2, 64), cached_v=z(1, 20, 2, 64),
+                                   moda_group_num=2)
+    with pytest.raises(AssertionError, match="same number of rows"):
+        moda_amd.parallel_moda_fwd(q, k, v, None, 0.125, cached_k=kd, cached_v=z(1, 16, 2, 64), moda_group_num=2)
+    with pytest.raises(AssertionError, match="k and v must agree"):
+        moda_amd.parallel_moda_fwd(q, k, z(1, 4, 2, 64), None, 0.125, moda_group_num=2)
+    # backward: o / do / lse of the wrong size
+    with pytest.raises(AssertionError, match="do must be"):
+        moda_amd.parallel_moda_bwd(q, k, v, o, None, lse, z(1, 8, 2, 64), 0.125, moda_group_num=2)
+    with pytest.raises(AssertionError, match="lse must be"):
+        moda_amd.parallel_moda_bwd(q, k, v, o, None, torch.zeros(1, 8, 2), do, 0.125, moda_group_num=2)
+    # depth-only: rows not a multiple of G, depth rows not T * L
+    with pytest.raises(AssertionError, match="multiple of moda_group_num"):
+        moda_amd.parallel_fda_fwd(z(1, 15, 2, 64), None, 0.125, cached_k=kd, cached_v=vd, moda_group_num=2)
+    with pytest.raises(AssertionError, match="depth rows must be T \\* L"):
+        moda_amd.parallel_fda_fwd(q, None, 0.125, cached_k=z(1, 20, 2, 64), cached_v=z(1, 20, 2, 64), moda_group_num=2)
+    # a consistent call gets as far as the device check
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        moda_amd.parallel_moda_fwd(q, k, v, None, 0.125, cached_k=kd, cached_v=vd, moda_group_num=2)
+    assert ops._check_shapes(_lib.CAUSAL, q, k, v, kd, vd, 2, o=o, do=do, lse=lse) == (8, 3)
+
+
+def test_depth_cache_append_checks_the_layer_against_the_cache():
+    import moda_amd
+
+    cache = moda_amd.DepthCache(2, 8, 3, 2, 64, torch.bfloat16, "cpu")
+    z = lambda *s, dt=torch.bfloat16: torch.zeros(*s, dtype=dt)
+    with pytest.raises(AssertionError, match="like the cache"):
+        cache.append(z(2, 9, 2, 64), z(2, 9, 2, 64))       # more tokens than the cache has
+    with pytest.raises(AssertionError, match="like the cache"):
+        cache.append(z(2, 8, 2, 128), z(2, 8, 2, 128))     # wider head dim
+    with pytest.raises(AssertionError, match="like the cache"):
+        cache.append(z(2, 8, 2, 64), z(2, 8, 4, 64))       # v with more heads
+    with pytest.raises(AssertionError, match="dtype"):
+        cache.append(z(2, 8, 2, 64, dt=torch.float16), z(2, 8, 2, 64, dt=torch.float16))
+    assert cache.n == 0
+    with pytest.raises(RuntimeError, match="no CPU path"):  # a matching layer reaches the device check
+        cache.append(z(2, 8, 2, 64), z(2, 8, 2, 64))
+    with pytest.raises(AssertionError, match="cache must be a contiguous"):
+        moda_amd.depth_cache._reorg_fwd([z(2, 8, 2, 64)], z(2, 16, 2, 64), 0, 3)
+
+
 def test_compat_package_reexports():
     import sys
 

@@ -223,6 +223,63 @@ def test_plain_gqa_matches_sdpa():
     assert torch.allclose(o, ref.permute(0, 2, 1, 3), atol=1e-12)
 
 
+def test_plain_gqa_lse_is_log2_of_the_row_sum():
+    """The comparator's second output: 2**lse must be the row sum of 2**(scale*log2(e)*<q,k>) over the visible
+    keys, computed here element by element without any library softmax."""
+    gen = torch.Generator().manual_seed(53)
+    B, T, Hq, Hkv, D = 2, 7, 6, 2, 8
+    q = torch.randn(B, T, Hq, D, generator=gen, dtype=D64)
+    k = torch.randn(B, T, Hkv, D, generator=gen, dtype=D64)
+    v = torch.randn(B, T, Hkv, D, generator=gen, dtype=D64)
+    _, lse = oracle.plain_gqa_dense(q, k, v, scale=0.37, dtype=D64)
+    assert lse.shape == (B, T, Hq)
+    for b in range(B):
+        for h in range(Hq):
+            for t in range(T):
+                tot = sum(math.exp(0.37 * float(q[b, t, h] @ k[b, j, h // (Hq // Hkv)])) for j in range(t + 1))
+                assert abs(2.0 ** float(lse[b, t, h]) - tot) <= 1e-9 * tot
+    # and it is the folded operator's lse after the kv-major regrouping of heads (query head hq -> kv head hq // G)
+    G = Hq // Hkv
+    qf = q.view(B, T, Hkv, G, D).permute(0, 1, 3, 2, 4).reshape(B, T * G, Hkv, D)
+    _, lse_f = oracle.moda_dense(qf, k, v, None, None, 0.37, G, "causal", dtype=D64)
+    assert torch.allclose(lse_f.view(B, T, G, Hkv).permute(0, 1, 3, 2).reshape(B, T, Hq), lse, atol=1e-12)
+
+
+@pytest.mark.parametrize("case", [(1, 24, 2, 8, 3, 2, "causal", 0), (1, 24, 1, 8, 2, 2, "chunk_visible", 4),
+                                  (2, 10, 2, 8, 3, 1, "noncausal", 0), (1, 12, 2, 8, 4, 2, "depth_only", 0)])
+def test_blockwise_token_range_and_rounded_o(case):
+    """The two optional branches of the tiled form.  token_range=(a, b): the rows of those tokens equal the full
+    evaluation's, and the key-side gradients equal those of a loss that only counts those rows (dO zeroed
+    elsewhere).  o_round_dtype: delta is taken from o rounded to that type, i.e. the result equals the
+    closed-form gradients with delta = sum(round(o) * do)."""
+    B, T, H, D, L, G, mode, cb = case
+    inp = _inputs(B, T, H, D, L, G, mode, seed=59)
+    a, b = (8, 20) if T >= 24 else (4, 8)
+    part = oracle.moda_blockwise_fwd_bwd(inp, 0.31, G, mode, cb, block_rows=4 * G, dtype=D64, token_range=(a, b))
+    masked = dict(inp)
+    masked["do"] = inp["do"].clone()
+    masked["do"][:, :a * G] = 0
+    masked["do"][:, b * G:] = 0
+    full = oracle.moda_dense_fwd_bwd(masked, 0.31, G, mode, cb, dtype=D64)
+    for n in ("o", "lse", "dq"):
+        assert torch.allclose(part[n][:, a * G:b * G], full[n][:, a * G:b * G], atol=1e-11), n
+    for n in ("dk", "dv", "dkd", "dvd"):
+        if full[n] is not None:
+            assert torch.allclose(part[n], full[n], atol=1e-11), n
+    # rounded o: compare with the explicit formulas evaluated densely
+    r = oracle.moda_blockwise_fwd_bwd(inp, 0.31, G, mode, cb, block_rows=4 * G, dtype=D64, o_round_dtype=torch.bfloat16)
+    exact = oracle.moda_dense_fwd_bwd(inp, 0.31, G, mode, cb, dtype=D64)
+    assert torch.allclose(r["o"], exact["o"], atol=1e-12)            # o itself is returned unrounded
+    # d(delta) = sum((round(o) - o) * do) per row shifts ds by -p * d(delta): dq changes by -d(delta) * scale * sum_j p_j key_j
+    ddelta = ((exact["o"].to(torch.bfloat16).to(D64) - exact["o"]) * inp["do"]).sum(-1)      # [B, rows, H]
+    assert ddelta.abs().max() > 0
+    q = inp["q"].clone().requires_grad_(True)
+    _, lse = oracle.moda_dense(q, inp["k"], inp["v"], inp["kd"], inp["vd"], 0.31, G, mode, cb, dtype=D64)
+    # sum_j p_j * scale * key_j = d(lse_natural)/dq, and lse is returned in base 2
+    (lse * math.log(2.0) * (-ddelta)).sum().backward()
+    assert torch.allclose(r["dq"], exact["dq"] + q.grad, atol=1e-10)
+
+
 def test_depth_cache_layout():
     layers = [torch.full((2, 3, 2, 4), float(l)) + torch.arange(3).view(1, 3, 1, 1) * 10 for l in range(5)]
     c = oracle.depth_cache_ref(layers)
