@@ -385,7 +385,7 @@ def main():
                                           stages=stages, out=state.get("grads"), ws=state.get("ws"), packed=packed)
 
         fwd()
-        state["ws"] = torch.empty(B * Hkv * G * T * 4 + 16, dtype=torch.uint8, device=dev)
+        state["ws"] = ops.bwd_workspace(mid, q, k, v, kd, vd, Garg, cb, packed=packed)
         bwd()
         for _ in range(warmup):
             fwd()

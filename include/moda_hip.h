@@ -132,9 +132,13 @@ int moda_hip_fwd(const moda_hip_desc* desc, const void* q, const void* k, const 
                  const void* kd, const void* vd, void* o, float* lse, void* stream);
 
 /*
- * Bytes of device workspace moda_hip_bwd needs (one fp32 per query row and
- * head: the row sum of o * do of moda_v14.py:525-539, kept in a form private to
- * the library).  Returns 0 for an invalid descriptor.
+ * Bytes of device workspace moda_hip_bwd asks for: one fp32 per query row and head (the row sum of
+ * o * do of moda_v14.py:525-539, kept in a form private to the library) and, for launches whose key
+ * tiles alone would leave compute units idle, fp32 partial sums of dk, dv per row segment (the role of
+ * the reference's dk_grouped / dv_grouped buffers, moda_v14.py:1715-1752; added up in a fixed order).
+ * A smaller workspace is accepted down to the row sums alone (B * H * G * T * 4 bytes; packed batch:
+ * H * G * total_tokens * 4): the backward then uses fewer row segments or none, which changes the fp32
+ * summation order of dk, dv but nothing else.  Returns 0 for an invalid descriptor.
  */
 size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* desc);
 
@@ -178,7 +182,9 @@ int moda_hip_bwd_stages(const moda_hip_desc* desc, const void* q, const void* k,
  * harnesses that forbid hipMalloc.  The row sums of o * do go to a workspace of
  * MODA_HIP_STATIC_WORKSPACE_BYTES that is part of the library's device image (one copy per GPU, held
  * until the process ends): problems with B * H * G * T fp32 values (packed batch: H * G * total_tokens)
- * beyond that size are rejected with MODA_HIP_ESTATIC.  Same kernels and results as moda_hip_bwd.
+ * beyond that size are rejected with MODA_HIP_ESTATIC.  Same kernels as moda_hip_bwd and the same results
+ * whenever moda_hip_bwd_workspace_bytes fits the built-in workspace (otherwise dk, dv are summed over fewer
+ * row segments, see there).
  * All calls on one GPU share the workspace: calls that may overlap on one GPU (different streams,
  * different host threads) race; serialise them or use moda_hip_bwd with private workspaces.  The first
  * call on a device looks the workspace address up (hipGetSymbolAddress, not a stream operation): under

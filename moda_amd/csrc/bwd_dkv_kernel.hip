@@ -40,8 +40,11 @@ __device__ __forceinline__ void unpack2<FP16>(int w, float& lo, float& hi) {
   hi = (float)v[1];
 }
 
-template <typename T, int HD, bool VARLEN>
+// SPLIT: the launch cuts the query rows of every sequence column tile into a.dkv_split segments (a variant of
+// its own: the extra index arithmetic costs the long-sequence instantiation scalar registers it cannot spare)
+template <typename T, int HD, bool VARLEN, bool SPLIT = false>
 __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
+  static_assert(!(VARLEN && SPLIT), "packed batches are not split");
   constexpr int BN = 128, BM = 64, KK = HD / 16, DB = HD / 32, NST = 3;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
@@ -63,9 +66,13 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   const int n_seq_tiles = a_in.has_seq ? (a_in.T + BN - 1) / BN : 0;
   SeqArgs<VARLEN> seq(a_in, b);
   const KArgs& a = seq.a;
-  const bool dep = ct >= n_seq_tiles;
+  // sequence tiles come `nseg` workgroups each (row segments of one column tile are neighbours in the grid, the
+  // heaviest column tile first), then the depth tiles
+  const int nseg = SPLIT ? a.dkv_split : 1;
+  const bool dep = ct >= n_seq_tiles * nseg;
   const int ncols = dep ? a.T * a.L : a.T;
-  int tile = dep ? ct - n_seq_tiles : ct;
+  const int seg = dep ? 0 : ct % nseg;
+  int tile = dep ? ct - n_seq_tiles * nseg : ct / nseg;
   if (VARLEN && !dep && a.causal) {
     // a causal sequence tile costs what lies behind it: count the grid's tiles from the end of the sequence, so
     // that tiles of equal cost of all sequences are dispatched together, the heaviest of the whole batch first
@@ -115,8 +122,13 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   int wg_lo, wg_hi, tmp;
   q_interval(c_first, wg_lo, tmp);
   q_interval(min(ncols, c_first + BN) - 1, tmp, wg_hi);
-  const int qt0 = wg_lo / BM;
-  const int nqt = (wg_hi + BM - 1) / BM - qt0;
+  int qt0 = wg_lo / BM;
+  int nqt = (wg_hi + BM - 1) / BM - qt0;
+  if (SPLIT && !dep) {  // this workgroup's share of the column tile's query tiles
+    const int lo = (int)((int64_t)nqt * seg / nseg), hi = (int)((int64_t)nqt * (seg + 1) / nseg);
+    qt0 += lo;
+    nqt = hi - lo;
+  }
   const int niter = nqt * a.hdiv;
 
   using Loader = AsyncTileLoader<HD, BM, 512>;
@@ -214,6 +226,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
     first_free_qt = ((min(ncols, c_first + BN) - 1) * a.Gf + BM - 1) / BM - qt0;
   else
     first_free_qt = 0;
+  if (SPLIT) first_free_qt = max(first_free_qt, 0);  // an upper row segment starts past the diagonal
   // the last sequence tile may hold padding columns: their K, V are zero, their results unused
 
   // role A, one tile: S = Q K^T, P = exp2(S c - lse) -> mailbox, dV^T += dO^T P
@@ -359,6 +372,25 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   else
     role_loop(std::true_type{});
 
+  if (SPLIT && !dep) {
+    // a row segment: fp32 partial sums, added up by dkv_reduce_kernel
+    if (valid) {
+      const int64_t plane = (int64_t)a.B * a.Hkv * a.T * HD;
+      float* outp = a.dkv_part + ((int64_t)(role_b ? 0 : 1) * nseg + seg) * plane +
+                    (((int64_t)b * a.Hkv + hkv) * a.T + c) * HD;
+      const float mul = role_b ? a.scale : 1.f;
+#pragma unroll
+      for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          f32x4 w;
+#pragma unroll
+          for (int j = 0; j < 4; j++) w[j] = acc[d][4 * i4 + j] * mul;
+          *reinterpret_cast<f32x4*>(outp + 32 * d + 8 * i4 + 4 * g) = w;
+        }
+    }
+    return;
+  }
   if (valid) {
     uint16_t* outp;
     float mul;
@@ -475,28 +507,77 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   *reinterpret_cast<i32x4*>(dv_out) = ov;
 }
 
+// Adds the fp32 partial sums of the row segments (in segment order: the result does not depend on which
+// workgroup finished first) and writes dk, dv in the tensor type.  One thread per 8 head-dim elements.
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void dkv_reduce_kernel(const KArgs a) {
+  constexpr int TPR = HD / 8;
+  const int64_t rows = (int64_t)a.B * a.Hkv * a.T;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = gid / TPR;
+  if (row >= rows) return;
+  const int sub = (int)(gid % TPR);
+  const int c = (int)(row % a.T);
+  const int bh = (int)(row / a.T);
+  const int b = bh / a.Hkv, hkv = bh % a.Hkv;
+  const int64_t plane = rows * HD;
+#pragma unroll
+  for (int which = 0; which < 2; which++) {  // 0: dk, 1: dv
+    const float* src = a.dkv_part + (int64_t)which * a.dkv_split * plane + row * HD + 8 * sub;
+    float s[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) s[i] = 0.f;
+    for (int sg = 0; sg < a.dkv_split; sg++) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(src + sg * plane);
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(src + sg * plane + 4);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        s[i] += lo[i];
+        s[4 + i] += hi[i];
+      }
+    }
+    i32x4 w;
+#pragma unroll
+    for (int i = 0; i < 4; i++) w[i] = pack2<T>(s[2 * i], s[2 * i + 1]);
+    uint16_t* outp = which == 0 ? a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t
+                                : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t;
+    *reinterpret_cast<i32x4*>(outp + 8 * sub) = w;
+  }
+}
+
 template <typename T, int HD>
 hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = 3 * 2 * 64 * HD * sizeof(uint16_t) + 2 * 4 * 4 * 64 * 16 + 3 * 2 * 64 * sizeof(float);
   static LdsAttrState attr;
   static LdsAttrState attr_packed;
+  static LdsAttrState attr_split;
+  const int nseg = a.cu ? 1 : a.dkv_split;
   const hipError_t ea =
-      a.cu ? allow_dynamic_lds(attr_packed, reinterpret_cast<const void*>(&dkv_kernel<T, HD, true>), smem)
-           : allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_kernel<T, HD, false>), smem);
+      a.cu       ? allow_dynamic_lds(attr_packed, reinterpret_cast<const void*>(&dkv_kernel<T, HD, true>), smem)
+      : nseg > 1 ? allow_dynamic_lds(attr_split, reinterpret_cast<const void*>(&dkv_kernel<T, HD, false, true>), smem)
+                 : allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_kernel<T, HD, false>), smem);
   if (ea != hipSuccess) return ea;
   // depth columns: vector kernel, except in chunk-visible mode where a column has up to G*Cb visible rows
   const bool depth_by_columns = a.L > 0 && !a.chunk;
   const int64_t n_seq_tiles = a.has_seq ? (a.T + 127) / 128 : 0;
   const int64_t n_dep_tiles = (a.L > 0 && !depth_by_columns) ? ((int64_t)a.T * a.L + 127) / 128 : 0;
-  const int64_t nblk = (n_seq_tiles + n_dep_tiles) * a.B * a.Hkv;
+  const int64_t nblk = (n_seq_tiles * nseg + n_dep_tiles) * a.B * a.Hkv;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   if (nblk > 0) {
     if (a.cu)
       hipLaunchKernelGGL((dkv_kernel<T, HD, true>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
+    else if (nseg > 1)
+      hipLaunchKernelGGL((dkv_kernel<T, HD, false, true>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
     else
       hipLaunchKernelGGL((dkv_kernel<T, HD, false>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    if (nseg > 1 && n_seq_tiles > 0) {
+      const int64_t nthreads = (int64_t)a.B * a.Hkv * a.T * (HD / 8);
+      hipLaunchKernelGGL((dkv_reduce_kernel<T, HD>), dim3((unsigned)((nthreads + 255) / 256)), dim3(256), 0, stream, a);
+      const hipError_t er = hipGetLastError();
+      if (er != hipSuccess) return er;
+    }
   }
   if (depth_by_columns && (int64_t)a.B * a.T > 0) {
     constexpr int CPB = 4 * (64 / (HD / 8));
@@ -511,6 +592,10 @@ template __global__ void depth_cols_kernel<BF16, 128>(const KArgs);
 template __global__ void depth_cols_kernel<BF16, 64>(const KArgs);
 template __global__ void depth_cols_kernel<FP16, 128>(const KArgs);
 template __global__ void depth_cols_kernel<FP16, 64>(const KArgs);
+template __global__ void dkv_kernel<BF16, 128, false, true>(const KArgs);
+template __global__ void dkv_kernel<BF16, 64, false, true>(const KArgs);
+template __global__ void dkv_kernel<FP16, 128, false, true>(const KArgs);
+template __global__ void dkv_kernel<FP16, 64, false, true>(const KArgs);
 template __global__ void dkv_kernel<BF16, 128, false>(const KArgs);
 template __global__ void dkv_kernel<BF16, 128, true>(const KArgs);
 template __global__ void dkv_kernel<BF16, 64, false>(const KArgs);

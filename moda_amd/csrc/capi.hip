@@ -86,6 +86,7 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   a.nqt = (a.Tq + 127) / 128;
   a.scale = d->scale;
   a.delta_pitch = a.Tq;
+  a.dkv_split = 1;
   if (d->cu_seqlens) {
     // packed batch: T is the longest sequence, the row axes hold total_tokens tokens
     if (d->total_tokens < d->T || ((uintptr_t)d->cu_seqlens % 4) != 0) return MODA_HIP_EINVAL;
@@ -95,6 +96,30 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
     a.delta_pitch = (int)(plain ? d->total_tokens : d->total_tokens * d->G);
   }
   return MODA_HIP_OK;
+}
+
+// Bytes of the row-sum part of the backward workspace, rounded up so that what follows stays aligned.
+size_t delta_bytes_exact(const KArgs& a) {
+  const size_t n = (a.cu ? (size_t)1 : (size_t)a.B) * a.Hq * a.delta_pitch * sizeof(float);
+  return n ? n : sizeof(float);
+}
+size_t delta_bytes(const KArgs& a) { return (delta_bytes_exact(a) + 255) / 256 * 256; }
+
+// Row segments per column tile of the sequence dK/dV kernel (see KArgs::dkv_split).  A launch whose column
+// tiles cannot give every compute unit two workgroups is cut further along the query rows, as long as a
+// segment keeps at least 16 query tiles.  Sized for the 256 compute units of a whole MI355X whatever the
+// partition mode, so that the workspace size depends on the descriptor alone.
+int desired_dkv_split(const moda_hip_desc* d, const KArgs& a) {
+  if (!use_mfma(d) || a.cu || !a.has_seq || a.T == 0) return 1;
+  const int64_t tiles = (int64_t)((a.T + 127) / 128) * a.B * a.Hkv;
+  const int64_t query_tiles = (a.Tq + 63) / 64;
+  int s = 1;
+  while (tiles * s < 512 && s < 8 && query_tiles / (2 * s) >= 16) s *= 2;
+  return s;
+}
+
+size_t dkv_part_bytes(const moda_hip_desc* d, const KArgs& a, int split) {
+  return split > 1 ? (size_t)2 * split * a.B * a.Hkv * a.T * d->D * sizeof(float) : 0;
 }
 
 // The current device must be a gfx950; reports its compute-unit count.  One entry per device is cached.
@@ -196,8 +221,8 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
 size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* d) {
   KArgs a;
   if (fill_geometry(d, a)) return 0;
-  const size_t n = (a.cu ? (size_t)1 : (size_t)a.B) * a.Hq * a.delta_pitch * sizeof(float);
-  return n ? n : sizeof(float);
+  const size_t part = dkv_part_bytes(d, a, desired_dkv_split(d, a));
+  return part ? delta_bytes(a) + part : delta_bytes_exact(a);
 }
 
 int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
@@ -210,9 +235,10 @@ int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const voi
 int moda_hip_bwd_static(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
                         const void* vd, const void* o, const float* lse, const void* d_o, void* dq, void* dk,
                         void* dv, void* dkd, void* dvd, void* stream) {
-  const size_t need = moda_hip_bwd_workspace_bytes(d);
-  if (need == 0) return MODA_HIP_EINVAL;
-  if (need > (size_t)MODA_HIP_STATIC_WORKSPACE_BYTES) return MODA_HIP_ESTATIC;
+  KArgs g;
+  const int grc = fill_geometry(d, g);
+  if (grc) return grc;
+  if (delta_bytes_exact(g) > (size_t)MODA_HIP_STATIC_WORKSPACE_BYTES) return MODA_HIP_ESTATIC;
   void* ws = nullptr;
   const int rc = static_workspace(&ws);
   if (rc) return rc;
@@ -261,7 +287,13 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
       MODA_REQ_ALIGN(dkd, d->dkd);
       MODA_REQ_ALIGN(dvd, d->dvd);
     }
-    if (!workspace || workspace_bytes < moda_hip_bwd_workspace_bytes(d)) return MODA_HIP_EWORKSPACE;
+    if (!workspace || workspace_bytes < delta_bytes_exact(a)) return MODA_HIP_EWORKSPACE;
+    // the row split of light launches uses what the workspace offers beyond the row sums: a caller that gives
+    // less than moda_hip_bwd_workspace_bytes asks for (moda_hip_bwd_static) gets fewer segments or none
+    int split = desired_dkv_split(d, a);
+    while (split > 1 && delta_bytes(a) + dkv_part_bytes(d, a, split) > workspace_bytes) split /= 2;
+    a.dkv_split = split;
+    a.dkv_part = (float*)((char*)workspace + delta_bytes(a));
   } else {
     return MODA_HIP_OK;
   }

@@ -277,6 +277,15 @@ def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages
     return dq, dk, dv, dkd, dvd
 
 
+def bwd_workspace(mode, q, k, v, kd, vd, G, chunk_tokens=0, packed=None) -> torch.Tensor:
+    """A workspace tensor of the size the backward asks for, for callers that reuse one across calls (``ws=``)."""
+    T, L = _check_shapes(mode, q, k, v, kd, vd, G)
+    kd_a, vd_a = (kd, vd) if L > 0 else (None, None)
+    d = _desc(mode, q, k, v, kd_a, vd_a, G, L, chunk_tokens, 1.0, packed=packed)
+    nbytes = _lib.load().moda_hip_bwd_workspace_bytes(ctypes.byref(d))
+    return torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=q.device)
+
+
 # ---------------------------------------------------------------------------
 # MoDA (causal / non-causal)  -- moda_v14.py
 # ---------------------------------------------------------------------------

@@ -54,13 +54,17 @@ def check(name, got, ref, dtype, what=""):
             f"at ref={ref.flatten()[i]:.4e} (atol={atol}, rtol={rtol}); max_abs={err.max():.4e}")
 
 
-def run_hip(inp, scale, G, mode, cb=0):
+def run_hip(inp, scale, G, mode, cb=0, row_sums_only=False):
+    """``row_sums_only``: give the backward a workspace that holds the row sums and nothing else, which keeps the
+    sequence dK/dV on the single-pass summation order (no row segments)."""
     from moda_amd import ops
 
     m = MODE_ID[mode]
     o, lse = ops._raw_fwd(m, inp["q"], inp["k"], inp["v"], inp["kd"], inp["vd"], scale, G, cb)
+    ws = torch.empty(max(4, 4 * inp["q"].shape[0] * inp["q"].shape[1] * inp["q"].shape[2]), dtype=torch.uint8,
+                     device=inp["q"].device) if row_sums_only else None
     dq, dk, dv, dkd, dvd = ops._raw_bwd(m, inp["q"], inp["k"], inp["v"], inp["kd"], inp["vd"], o, lse, inp["do"],
-                                        scale, G, cb)
+                                        scale, G, cb, ws=ws)
     return {"o": o, "lse": lse, "dq": dq, "dk": dk, "dv": dv, "dkd": dkd, "dvd": dvd}
 
 
@@ -702,6 +706,45 @@ def test_depth_gradients_accumulate_over_layers(gpu_device, case):
         assert rel <= 1e-2, (name, float(rel))
 
 
+@pytest.mark.parametrize("case", [
+    # (B, T, H, D, L, G, mode, dtype)
+    (1, 1024, 1, 64, 2, 4, "causal", torch.bfloat16),      # 8 key tiles, four row segments each
+    (1, 1100, 2, 128, 0, 2, "causal", torch.float16),      # ragged last tile, two segments
+    (1, 1024, 2, 128, 1, 2, "noncausal", torch.bfloat16),
+    (1, 1024, 1, 128, 3, 4, "chunk_visible", torch.bfloat16),
+])
+def test_row_split_sequence_gradients(gpu_device, case):
+    """Launches with few key tiles cut every tile's query rows into segments that leave fp32 partial sums for a
+    second kernel to add (shapes chosen so that the split is taken).  Checked against the oracle like every other
+    case, and against the unsplit evaluation the same library gives with a workspace that only holds the row sums."""
+    import ctypes
+
+    from moda_amd import _lib, ops
+
+    B, T, H, D, L, G, mode, dtype = case
+    say(f"CASE row-split {case}")
+    cb = 16 if mode == "chunk_visible" else 0
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=83, dtype=dtype, std=0.5)
+    sc = D ** -0.5
+    ref = oracle.moda_dense_fwd_bwd(inp, sc, G, mode, cb)
+    dev = to_dev(inp, gpu_device)
+    m = MODE_ID[mode]
+    ws = ops.bwd_workspace(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], G, cb)
+    rows_only = B * H * T * G * 4
+    assert ws.numel() > rows_only + 256, "this shape was meant to take the row split"
+    got = run_hip(dev, sc, G, mode, cb)
+    compare_all(got, ref, dtype, f"row-split {case}")
+    small = torch.empty(rows_only, dtype=torch.uint8, device=gpu_device)
+    dq, dk, dv, dkd, dvd = ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], got["o"], got["lse"],
+                                        dev["do"], sc, G, cb, ws=small)
+    assert torch.equal(dq, got["dq"])
+    check("dk", dk, ref["dk"], dtype, "unsplit")
+    check("dv", dv, ref["dv"], dtype, "unsplit")
+    # the two summation orders agree to a rounding of the 16-bit result
+    for a, b_ in ((dk, got["dk"]), (dv, got["dv"])):
+        assert ((a.float() - b_.float()).abs() <= 2.0 ** -7 * b_.float().abs() + 1e-3).all()
+
+
 def test_hip_graph_capture_and_replay(gpu_device):
     """Forward + backward captured in a HIP graph (the library allocates nothing and clears nothing, so
     every launch is capturable) and replayed with new inputs; every replay is checked against eager."""
@@ -859,7 +902,8 @@ def test_packed_batch_equals_separate_calls_bitwise(gpu_device):
         a, b = cu[i], cu[i + 1]
         part = {n: inp[n][:, a * m:b * m] for n, m in mult.items()}
         part["do"] = inp["do"][:, a * G:b * G]
-        one = run_hip(part, D ** -0.5, G, "causal")
+        # (the packed launch sums dk, dv in one pass per key tile: ask the separate calls for the same order)
+        one = run_hip(part, D ** -0.5, G, "causal", row_sums_only=True)
         assert torch.equal(o[:, a * G:b * G], one["o"]) and torch.equal(lse[:, a * G:b * G], one["lse"]), i
         for n, key in (("q", "dq"), ("k", "dk"), ("v", "dv"), ("kd", "dkd"), ("vd", "dvd")):
             assert torch.equal(leaf[n].grad[:, a * mult[n]:b * mult[n]], one[key]), (i, n)

@@ -91,6 +91,40 @@ def test_static_workspace_backward_matches_and_survives_a_smaller_second_call(gp
     _both_backwards(dev, 1, 96, 2, 64, 2, 4, "chunk_visible", torch.float16, cb=16, seed=3)
 
 
+def test_static_workspace_with_fewer_row_segments(gpu_device):
+    """A shape for which moda_hip_bwd asks for more workspace than the built-in one holds (fp32 partial sums of
+    dk, dv per row segment): the allocation-free entry point then sums over fewer segments, which may move the
+    last bit of dk, dv and nothing else."""
+    from moda_amd import _lib, ops
+
+    lib = _lib.load()
+    dev = gpu_device
+    B, T, H, D, L, G = 2, 2048, 4, 128, 1, 4
+    say(f"no-alloc backward, fewer row segments: B={B} T={T} H={H} D={D} L={L} G={G}")
+    gen = torch.Generator(device=dev).manual_seed(3)
+    rn = lambda *s: (0.5 * torch.randn(*s, generator=gen, device=dev)).bfloat16()
+    q, k, v, kd, vd, do = rn(B, T * G, H, D), rn(B, T, H, D), rn(B, T, H, D), rn(B, T * L, H, D), rn(B, T * L, H, D), \
+        rn(B, T * G, H, D)
+    sc = D ** -0.5
+    o, lse = ops._raw_fwd(_lib.CAUSAL, q, k, v, kd, vd, sc, G)
+    ws = ops.bwd_workspace(_lib.CAUSAL, q, k, v, kd, vd, G)
+    assert ws.numel() > _lib.STATIC_WORKSPACE_BYTES
+    a = ops._raw_bwd(_lib.CAUSAL, q, k, v, kd, vd, o, lse, do, sc, G, ws=ws)
+    b = tuple(torch.full_like(x, float("nan")) for x in a)
+    d = ops._desc(_lib.CAUSAL, q, k, v, kd, vd, G, L, 0, sc, o=o, do=do, dq=b[0], dk=b[1], dv=b[2], dkd=b[3], dvd=b[4])
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    rc = lib.moda_hip_bwd_static(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kd), _ptr(vd), _ptr(o), _ptr(lse),
+                                 _ptr(do), _ptr(b[0]), _ptr(b[1]), _ptr(b[2]), _ptr(b[3]), _ptr(b[4]), stream)
+    assert rc == 0, lib.moda_hip_strerror(rc)
+    for i in (0, 3, 4):  # dq, dkd, dvd: untouched by the split
+        assert torch.equal(a[i].view(torch.int16), b[i].view(torch.int16))
+    for i in (1, 2):     # dk, dv: same sums in another order
+        x, y = a[i].float(), b[i].float()
+        assert torch.isfinite(y).all()
+        assert bool(((x - y).abs() <= 2e-2 + 2.0 ** -7 * x.abs()).all())
+        assert ((x - y).norm() / x.norm()).item() <= 4e-3
+
+
 def test_static_workspace_rejects_oversized_problems(gpu_device):
     from moda_amd import _lib
 
