@@ -26,20 +26,6 @@
 
 namespace moda {
 
-template <typename T>
-__device__ __forceinline__ void unpack2(int w, float& lo, float& hi);
-template <>
-__device__ __forceinline__ void unpack2<BF16>(int w, float& lo, float& hi) {
-  lo = __builtin_bit_cast(float, w << 16);
-  hi = __builtin_bit_cast(float, w & 0xffff0000);
-}
-template <>
-__device__ __forceinline__ void unpack2<FP16>(int w, float& lo, float& hi) {
-  const f16x2 v = __builtin_bit_cast(f16x2, w);
-  lo = (float)v[0];
-  hi = (float)v[1];
-}
-
 // SPLIT: the launch cuts the query rows of every sequence column tile into a.dkv_split segments (a variant of
 // its own: the extra index arithmetic costs the long-sequence instantiation scalar registers it cannot spare)
 template <typename T, int HD, bool VARLEN, bool SPLIT = false>
@@ -415,6 +401,181 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   }
 }
 
+// Depth columns in chunk-visible mode when a chunk's query rows fit one 64-row tile (the reference's only
+// shipped geometry: 64 rows per chunk, moda_v16.py:581-585, 1632-1834).  A depth slot is then seen by rows of ONE
+// query tile only, so the column-tile kernel above would run a single trip per workgroup and spend its time on
+// start-up latency.  Here a workgroup of four waves owns a whole CHUNK: the chunk's Q, dO, lse and delta are
+// staged once, then every wave takes 32-column blocks of the chunk's depth slots and does both halves of the
+// work itself -- S, P, dV^T with the slots' K rows in registers, then dP, dS, dK^T with their V rows -- with P kept
+// in registers in between (no mailbox, no barrier after the staging).  The slots' K/V rows come in and the
+// gradient rows go out through a wave-private 32-row tile, so that every global access covers whole rows
+// (operand-shaped accesses straight to global memory touch 32 rows per instruction and are bound by the
+// request rate).  Two workgroups share a compute unit.
+template <typename T, int HD, bool VARLEN>
+__global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
+  constexpr int BM = 64, KK = HD / 16, DB = HD / 32;
+  constexpr int CH = HD / 8, RPW = 64 / CH, NPASS = 32 / RPW;  // 16-byte chunks per row, rows per wave-wide access
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  lds_ptr Qs = (lds_ptr)smem_raw;
+  lds_ptr dOs = Qs + BM * HD;
+  const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  lds_ptr wt = dOs + BM * HD + wave * (32 * HD);                           // this wave's private tile
+  MODA_LDS float* stat = (MODA_LDS float*)(dOs + BM * HD + 4 * 32 * HD);    // lse[BM], then minus delta[BM]
+
+  const int BHk = a_in.B * a_in.Hkv;
+  const int bh = blockIdx.x % BHk;
+  const int chunk = blockIdx.x / BHk;
+  int b = bh / a_in.Hkv;
+  const int hkv = bh % a_in.Hkv;
+  SeqArgs<VARLEN> seq(a_in, b);
+  const KArgs& a = seq.a;
+  const int t0 = chunk * a.Cb;
+  if (t0 >= a.T) return;  // a chunk beyond this sequence of a variable-length batch
+  const int t1 = min(a.T, t0 + a.Cb);
+  const int r0 = t0 * a.Gf, r_end = t1 * a.Gf;  // the chunk's query rows (at most BM)
+
+  using Loader = AsyncTileLoader<HD, BM, 256>;
+  Loader ld;
+  ld.init(tid);
+  ld.load(Qs, a.q + b * a.sq.b + hkv * a.sq.h, a.sq.t, r0, r_end);
+  ld.load(dOs, a.d_o + b * a.sdo.b + hkv * a.sdo.h, a.sdo.t, r0, r_end);
+  if (tid < BM) {
+    const int r = r0 + tid;
+    const bool in = r < r_end;
+    stat[tid] = in ? a.lse[((int64_t)b * a.Tq + r) * a.Hq + hkv] : 0.f;
+    stat[BM + tid] = in ? a.delta[((int64_t)b * a.Hq + hkv) * (VARLEN ? a.delta_pitch : a.Tq) + r] : 0.f;
+  }
+  Loader::wait_all();
+  __syncthreads();
+
+  const float sc = a.scale * kLog2e;
+  OperandAddr<HD> oa;
+  oa.init(lane);
+  const int c_end = t1 * a.L;
+  const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
+  const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
+  const int prow = lane / CH, pch = lane % CH;  // this lane's row within a pass over the private tile, its physical chunk
+  // rows [cb, cb + 32) of a depth tensor -> the private tile (rows past the chunk's last column arrive as zeros)
+  auto fetch = [&](const uint16_t* base, int64_t stride, int cb) {
+    const int nrows = min(32, c_end - cb);
+    const i32x4 rs = rsrc_words(base + (int64_t)cb * stride, (uint32_t)nrows * (uint32_t)stride * 2u);
+#pragma unroll
+    for (int i = 0; i < NPASS; i++) {
+      const int row = i * RPW + prow;
+      lds_dma<16>(rs, lds_addr(wt + i * 512), row * (int)stride * 2 + (pch ^ Tile<HD>::swz(row)) * 16, 0);
+    }
+  };
+  auto landed = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    asm volatile("" ::: "memory");
+  };
+  auto reads_done = [&]() {  // every LDS read of this wave has returned: the tile may be overwritten
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    asm volatile("" ::: "memory");
+  };
+  // 32 gradient rows from the accumulators (one column per lane) through the private tile to global memory
+  auto store = [&](const f32x16 (&acc)[DB], uint16_t* base, int64_t stride, int cb, float mul) {
+    reads_done();
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        i32x2 w;
+        w[0] = pack2<T>(acc[d][4 * i4 + 0] * mul, acc[d][4 * i4 + 1] * mul);
+        w[1] = pack2<T>(acc[d][4 * i4 + 2] * mul, acc[d][4 * i4 + 3] * mul);
+        *reinterpret_cast<MODA_LDS i32x2*>(wt + Tile<HD>::off(n, 4 * d + i4) + 4 * g) = w;
+      }
+#pragma unroll
+    for (int i = 0; i < NPASS; i++) {
+      const int row = i * RPW + prow;
+      const i32x4 val = *reinterpret_cast<MODA_LDS const i32x4*>(wt + i * 512 + lane * 8);
+      if (cb + row < c_end)
+        *reinterpret_cast<i32x4*>(base + (int64_t)(cb + row) * stride + (pch ^ Tile<HD>::swz(row)) * 8) = val;
+    }
+  };
+
+  for (int cb = t0 * a.L + wave * 32; cb < c_end; cb += 128) {
+    const int c = cb + n;
+    // the column's visible rows: from its owner token's first row to the end of the chunk
+    const int qlo = c < c_end ? (c / a.L) * a.Gf : r_end;
+    reads_done();
+    fetch(kdp, a.skd.t, cb);
+    landed();
+    i32x4 Sr[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) Sr[kk] = oa.row_operand(wt, 0, kk);
+    reads_done();
+    fetch(vdp, a.svd.t, cb);  // the V rows travel while the probabilities are computed
+    // S = Q K^T, P = exp2(S c - lse) on the visible rows
+    f32x16 s[2];
+    mfma_rows<T, HD, 2, 4>(oa, Qs, Sr, s);
+#pragma unroll
+    for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(stat + 32 * bb + 8 * i4 + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const int qr = r0 + 32 * bb + 8 * i4 + 4 * g + j;
+          const float p = fast_exp2(__builtin_fmaf(s[bb][4 * i4 + j], sc, -lv[j]));
+          s[bb][4 * i4 + j] = (qr >= qlo && qr < r_end) ? p : 0.f;
+        }
+      }
+    i32x4 P[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+    landed();
+    i32x4 Vr[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) Vr[kk] = oa.row_operand(wt, 0, kk);
+    {  // dV^T = dO^T P
+      f32x16 acc[DB];
+#pragma unroll
+      for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[d][i] = 0.f;
+      TrPipe<T, HD, 4, 2> dvp;
+      dvp.prefetch(oa, dOs);
+      dvp.run(oa, dOs, P, acc);
+      store(acc, a.dvd + b * a.sdvd.b + hkv * a.sdvd.h, a.sdvd.t, cb, 1.f);
+    }
+    {  // dP - delta = dO V^T (accumulators start from minus delta), dS = P (dP - delta), dK^T = Q^T dS
+      f32x16 dp[2];
+#pragma unroll
+      for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          const f32x4 dl = *reinterpret_cast<MODA_LDS const f32x4*>(stat + BM + 32 * bb + 8 * i4 + 4 * g);
+#pragma unroll
+          for (int j = 0; j < 4; j++) dp[bb][4 * i4 + j] = dl[j];
+        }
+      mfma_rows_acc<T, HD, 2, 4>(oa, dOs, Vr, dp);
+      i32x4 DS[4];
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        const int bb = ks >> 1;
+        float p[8];
+#pragma unroll
+        for (int w = 0; w < 4; w++) unpack2<T>(P[ks][w], p[2 * w], p[2 * w + 1]);
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+          DS[ks][w] = pack2<T>(p[2 * w] * dp[bb][8 * (ks & 1) + 2 * w], p[2 * w + 1] * dp[bb][8 * (ks & 1) + 2 * w + 1]);
+      }
+      f32x16 acc[DB];
+#pragma unroll
+      for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[d][i] = 0.f;
+      TrPipe<T, HD, 4, 2> dkp;
+      dkp.prefetch(oa, Qs);
+      dkp.run(oa, Qs, DS, acc);
+      store(acc, a.dkd + b * a.sdkd.b + hkv * a.sdkd.h, a.sdkd.t, cb, a.scale);
+    }
+  }
+}
+
 // Depth columns outside chunk-visible mode (moda_v14.py:1251-1454, fda_v12.py:646-860): a depth slot is seen
 // by the G query rows of its own token only, so its gradients are 2*G dot products and 2*G scaled row
 // additions of length D -- far too little to fill a 64 x 128 MFMA tile, and on short sequences the
@@ -560,7 +721,9 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   // depth columns: vector kernel, except in chunk-visible mode where a column has up to G*Cb visible rows
   const bool depth_by_columns = a.L > 0 && !a.chunk;
   const int64_t n_seq_tiles = a.has_seq ? (a.T + 127) / 128 : 0;
-  const int64_t n_dep_tiles = (a.L > 0 && !depth_by_columns) ? ((int64_t)a.T * a.L + 127) / 128 : 0;
+  // chunk-visible depth columns: by whole chunks when a chunk's rows fit one query tile, else as column tiles
+  const bool depth_by_chunks = a.L > 0 && a.chunk && (int64_t)a.Cb * a.Gf <= 64;
+  const int64_t n_dep_tiles = (a.L > 0 && a.chunk && !depth_by_chunks) ? ((int64_t)a.T * a.L + 127) / 128 : 0;
   const int64_t nblk = (n_seq_tiles * nseg + n_dep_tiles) * a.B * a.Hkv;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   if (nblk > 0) {
@@ -578,6 +741,20 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
       const hipError_t er = hipGetLastError();
       if (er != hipSuccess) return er;
     }
+  }
+  if (depth_by_chunks && (int64_t)a.B * a.T > 0) {
+    constexpr size_t csmem = (2 * 64 + 4 * 32) * HD * sizeof(uint16_t) + 2 * 64 * sizeof(float);
+    const int64_t nx = (((int64_t)a.T + a.Cb - 1) / a.Cb) * a.B * a.Hkv;
+    if (nx >= (1ll << 31)) return hipErrorInvalidValue;
+    static LdsAttrState cattr, cattr_packed;
+    const hipError_t ec =
+        a.cu ? allow_dynamic_lds(cattr_packed, reinterpret_cast<const void*>(&chunk_depth_kernel<T, HD, true>), csmem)
+             : allow_dynamic_lds(cattr, reinterpret_cast<const void*>(&chunk_depth_kernel<T, HD, false>), csmem);
+    if (ec != hipSuccess) return ec;
+    if (a.cu)
+      hipLaunchKernelGGL((chunk_depth_kernel<T, HD, true>), dim3((unsigned)nx), dim3(256), csmem, stream, a);
+    else
+      hipLaunchKernelGGL((chunk_depth_kernel<T, HD, false>), dim3((unsigned)nx), dim3(256), csmem, stream, a);
   }
   if (depth_by_columns && (int64_t)a.B * a.T > 0) {
     constexpr int CPB = 4 * (64 / (HD / 8));

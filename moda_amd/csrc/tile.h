@@ -76,6 +76,21 @@ __device__ __forceinline__ int pack2<FP16>(float a, float b) {
   return __builtin_bit_cast(int, v);
 }
 
+// One packed pair of 16-bit values -> fp32.
+template <typename T>
+__device__ __forceinline__ void unpack2(int w, float& lo, float& hi);
+template <>
+__device__ __forceinline__ void unpack2<BF16>(int w, float& lo, float& hi) {
+  lo = __builtin_bit_cast(float, w << 16);
+  hi = __builtin_bit_cast(float, w & 0xffff0000);
+}
+template <>
+__device__ __forceinline__ void unpack2<FP16>(int w, float& lo, float& hi) {
+  const f16x2 v = __builtin_bit_cast(f16x2, w);
+  lo = (float)v[0];
+  hi = (float)v[1];
+}
+
 // Eight consecutive accumulator registers -> one MFMA B operand (k slots 0..7).
 template <typename T>
 __device__ __forceinline__ i32x4 pack8(const f32x16& x, int first) {
