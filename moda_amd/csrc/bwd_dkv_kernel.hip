@@ -81,7 +81,9 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       i32x4 z = {0, 0, 0, 0};
-      Sr[kk] = (valid && !empty_slot) ? *reinterpret_cast<const i32x4*>(src + (int64_t)c * st + 16 * kk + 8 * g) : z;
+      Sr[kk] = (valid && !empty_slot && 16 * kk + 8 * g < a.D)
+                   ? *reinterpret_cast<const i32x4*>(src + (int64_t)c * st + 16 * kk + 8 * g)
+                   : z;
     }
   }
 
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   using Loader = AsyncTileLoader<HD, BM, 512>;
   static_assert(Loader::N == HD / 64, "one or two wave-wide loads per tile and wave");
   Loader ld;
-  ld.init(tid);
+  ld.init(tid, a.D);
   // Producer.  The global -> LDS loads of one tile are NOT issued back to back: forty wave-wide
   // loads arriving at once queue up in the CU's address unit and every wave would sit on its issue
   // for hundreds of cycles.  prep() fixes the descriptors of the next tile (wave-uniform, scalar
@@ -131,8 +133,8 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   // wave's statistic) that step down one tile per call: the scalar unit then has a few adds per trip
   // instead of a dozen dependent 64-bit multiplies.
   const uint32_t q_row_bytes = (uint32_t)a.sq.t * 2u, do_row_bytes = (uint32_t)a.sdo.t * 2u;
-  const int voff_q = ld.row_in_pass * (int)q_row_bytes + ld.gchunk * 16;
-  const int voff_do = ld.row_in_pass * (int)do_row_bytes + ld.gchunk * 16;
+  const int voff_q = ld.lane_offset((int)q_row_bytes);
+  const int voff_do = ld.lane_offset((int)do_row_bytes);
   // wave 0 fetches lse ([B, Tq, Hq]: one dword every Hq), wave 1 delta ([B, Hq, Tq]: contiguous)
   const int voff_stat = wave == 0 ? lane * a.Hq * 4 : lane * 4;
   const uint32_t stat_row_bytes = wave == 0 ? (uint32_t)a.Hq * 4u : 4u;
@@ -396,7 +398,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
         i32x2 w;
         w[0] = pack2<T>(acc[d][4 * i4 + 0] * mul, acc[d][4 * i4 + 1] * mul);
         w[1] = pack2<T>(acc[d][4 * i4 + 2] * mul, acc[d][4 * i4 + 3] * mul);
-        *reinterpret_cast<i32x2*>(outp + 32 * d + 8 * i4 + 4 * g) = w;
+        if (32 * d + 8 * i4 + 4 * g < a.D) *reinterpret_cast<i32x2*>(outp + 32 * d + 8 * i4 + 4 * g) = w;
       }
   }
 }
@@ -437,7 +439,7 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
 
   using Loader = AsyncTileLoader<HD, BM, 256>;
   Loader ld;
-  ld.init(tid);
+  ld.init(tid, a.D);
   ld.load(Qs, a.q + b * a.sq.b + hkv * a.sq.h, a.sq.t, r0, r_end);
   ld.load(dOs, a.d_o + b * a.sdo.b + hkv * a.sdo.h, a.sdo.t, r0, r_end);
   if (tid < BM) {
@@ -463,7 +465,8 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
 #pragma unroll
     for (int i = 0; i < NPASS; i++) {
       const int row = i * RPW + prow;
-      lds_dma<16>(rs, lds_addr(wt + i * 512), row * (int)stride * 2 + (pch ^ Tile<HD>::swz(row)) * 16, 0);
+      const int lch = pch ^ Tile<HD>::swz(row);  // chunks beyond the head dim: out of range, filled with zeros
+      lds_dma<16>(rs, lds_addr(wt + i * 512), lch * 8 < a.D ? row * (int)stride * 2 + lch * 16 : Loader::kPadOffset, 0);
     }
   };
   auto landed = [&]() {
@@ -491,8 +494,9 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
     for (int i = 0; i < NPASS; i++) {
       const int row = i * RPW + prow;
       const i32x4 val = *reinterpret_cast<MODA_LDS const i32x4*>(wt + i * 512 + lane * 8);
-      if (cb + row < c_end)
-        *reinterpret_cast<i32x4*>(base + (int64_t)(cb + row) * stride + (pch ^ Tile<HD>::swz(row)) * 8) = val;
+      const int lch = pch ^ Tile<HD>::swz(row);
+      if (cb + row < c_end && lch * 8 < a.D)
+        *reinterpret_cast<i32x4*>(base + (int64_t)(cb + row) * stride + lch * 8) = val;
     }
   };
 
@@ -599,15 +603,17 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   const int w = (int)(c / a.L), slot = (int)(c - (int64_t)w * a.L);
   uint16_t* dk_out = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + c * a.sdkd.t + 8 * sub;
   uint16_t* dv_out = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + c * a.sdvd.t + 8 * sub;
+  const bool in_dim = 8 * sub < a.D;  // lanes past the tensors' head dim carry zeros and store nothing
   if (slot >= a.Lv) {  // a slot without data: zero gradient, or (accumulating) somebody else's sum to leave alone
-    if (a.accum_depth) return;
+    if (a.accum_depth || !in_dim) return;
     const i32x4 z = {0, 0, 0, 0};
     *reinterpret_cast<i32x4*>(dk_out) = z;
     *reinterpret_cast<i32x4*>(dv_out) = z;
     return;
   }
   auto load8 = [&](const uint16_t* p, float (&f)[8]) {
-    const i32x4 v = *reinterpret_cast<const i32x4*>(p);
+    const i32x4 zero = {0, 0, 0, 0};
+    const i32x4 v = in_dim ? *reinterpret_cast<const i32x4*>(p) : zero;
 #pragma unroll
     for (int i = 0; i < 4; i++) unpack2<T>(v[i], f[2 * i], f[2 * i + 1]);
   };
@@ -664,8 +670,10 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
     ok[i] = pack2<T>(dk[2 * i], dk[2 * i + 1]);
     ov[i] = pack2<T>(dv[2 * i], dv[2 * i + 1]);
   }
-  *reinterpret_cast<i32x4*>(dk_out) = ok;
-  *reinterpret_cast<i32x4*>(dv_out) = ov;
+  if (in_dim) {
+    *reinterpret_cast<i32x4*>(dk_out) = ok;
+    *reinterpret_cast<i32x4*>(dv_out) = ov;
+  }
 }
 
 // Adds the fp32 partial sums of the row segments (in segment order: the result does not depend on which
@@ -702,7 +710,7 @@ __global__ __launch_bounds__(256) void dkv_reduce_kernel(const KArgs a) {
     for (int i = 0; i < 4; i++) w[i] = pack2<T>(s[2 * i], s[2 * i + 1]);
     uint16_t* outp = which == 0 ? a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t
                                 : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t;
-    *reinterpret_cast<i32x4*>(outp + 8 * sub) = w;
+    if (8 * sub < a.D) *reinterpret_cast<i32x4*>(outp + 8 * sub) = w;
   }
 }
 

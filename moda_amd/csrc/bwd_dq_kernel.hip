@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a_in) {
   const int r = rb * RPB + tid / TPR;
   const int c = (tid % TPR) * 8;
   float acc = 0.f;
-  if (r < a.Tq) {
+  if (r < a.Tq && c < a.D) {
     const uint16_t* op = a.o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + c;
     const uint16_t* dp = a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + c;
     const typename T::vec8 ov = *reinterpret_cast<const typename T::vec8*>(op);
@@ -82,8 +82,9 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       i32x4 z = {0, 0, 0, 0};
-      Qr[kk] = valid ? *reinterpret_cast<const i32x4*>(qp + 16 * kk) : z;
-      dOr[kk] = valid ? *reinterpret_cast<const i32x4*>(dop + 16 * kk) : z;
+      const bool in = valid && 16 * kk + 8 * g < a.D;
+      Qr[kk] = in ? *reinterpret_cast<const i32x4*>(qp + 16 * kk) : z;
+      dOr[kk] = in ? *reinterpret_cast<const i32x4*>(dop + 16 * kk) : z;
     }
     if (valid) {
       lse = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq];
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   typedef AsyncTileLoader<HD, BN, NT> Loader;
   constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
   Loader ld;
-  ld.init(tid);
+  ld.init(tid, a.D);
   // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
   // producer reaches the first depth tile
   typename Loader::Source srcK, srcV;
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
         i32x2 w;
         w[0] = pack2<T>(dq[d][4 * i4 + 0] * a.scale, dq[d][4 * i4 + 1] * a.scale);
         w[1] = pack2<T>(dq[d][4 * i4 + 2] * a.scale, dq[d][4 * i4 + 3] * a.scale);
-        *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
+        if (32 * d + 8 * i4 + 4 * g < a.D) *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
       }
   }
 }

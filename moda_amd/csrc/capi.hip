@@ -43,10 +43,13 @@ bool row_stride_ok(const moda_hip_strides& s, int esize) { return s.t >= 0 && s.
 
 int value_dim(const moda_hip_desc* d) { return (int)(d->Dv > 0 ? d->Dv : d->D); }
 
+// The matrix-core kernels exist for tile widths 64 and 128; any 16-bit head dim that is a multiple of 8 (whole
+// 16-byte chunks) up to 128 runs on the next width, zero-padded inside the kernels.
 bool use_mfma(const moda_hip_desc* d) {
-  return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && (d->D == 64 || d->D == 128) &&
+  return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && d->D % 8 == 0 && d->D <= 128 &&
          value_dim(d) == d->D;
 }
+int tile_width(const moda_hip_desc* d) { return d->D <= 64 ? 64 : 128; }
 
 // Validates the descriptor and fills the geometry part of KArgs.
 int fill_geometry(const moda_hip_desc* d, KArgs& a) {
@@ -72,6 +75,7 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   a.B = (int)d->B;
   a.T = (int)d->T;
   a.Hkv = (int)d->H;
+  a.D = (int)d->D;
   a.Tq = plain ? (int)d->T : (int)(d->T * d->G);
   a.Gf = plain ? 1 : (int)d->G;
   a.Hq = plain ? (int)(d->H * d->G) : (int)d->H;
@@ -119,7 +123,7 @@ int desired_dkv_split(const moda_hip_desc* d, const KArgs& a) {
 }
 
 size_t dkv_part_bytes(const moda_hip_desc* d, const KArgs& a, int split) {
-  return split > 1 ? (size_t)2 * split * a.B * a.Hkv * a.T * d->D * sizeof(float) : 0;
+  return split > 1 ? (size_t)2 * split * a.B * a.Hkv * a.T * tile_width(d) * sizeof(float) : 0;
 }
 
 // The current device must be a gfx950; reports its compute-unit count.  One entry per device is cached.
@@ -213,7 +217,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
   a.skd = cvt(d->kd);
   a.svd = cvt(d->vd);
   a.so = cvt(d->o);
-  hipError_t e = use_mfma(d) ? moda::launch_fwd(a, d->dtype, (int)d->D, (hipStream_t)stream)
+  hipError_t e = use_mfma(d) ? moda::launch_fwd(a, d->dtype, tile_width(d), (hipStream_t)stream)
                              : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 0, (hipStream_t)stream);
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }
@@ -327,9 +331,9 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = hipSuccess;
   if (use_mfma(d)) {
-    if (stages & MODA_HIP_STAGE_DELTA) e = moda::launch_delta(a, d->dtype, (int)d->D, s);
-    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ)) e = moda::launch_dq(a, d->dtype, (int)d->D, s);
-    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_dkv(a, d->dtype, (int)d->D, s);
+    if (stages & MODA_HIP_STAGE_DELTA) e = moda::launch_delta(a, d->dtype, tile_width(d), s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ)) e = moda::launch_dq(a, d->dtype, tile_width(d), s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_dkv(a, d->dtype, tile_width(d), s);
   } else {
     // the generic kernels recompute delta inline; the DELTA stage is a no-op for them
     if (stages & MODA_HIP_STAGE_DQ) e = moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 1, s);

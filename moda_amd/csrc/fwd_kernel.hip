@@ -62,7 +62,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       i32x4 z = {0, 0, 0, 0};
-      Qr[kk] = valid ? *reinterpret_cast<const i32x4*>(qp + 16 * kk) : z;
+      Qr[kk] = (valid && 16 * kk + 8 * g < a.D) ? *reinterpret_cast<const i32x4*>(qp + 16 * kk) : z;
     }
   }
 
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   typedef AsyncTileLoader<HD, BN, NT> Loader;
   constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
   Loader ld;
-  ld.init(tid);
+  ld.init(tid, a.D);
   // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
   // producer reaches the first depth tile
   typename Loader::Source srcK, srcV;
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         i32x2 w;
         w[0] = pack2<T>(o[d][4 * i4 + 0] * inv, o[d][4 * i4 + 1] * inv);
         w[1] = pack2<T>(o[d][4 * i4 + 2] * inv, o[d][4 * i4 + 3] * inv);
-        *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
+        if (32 * d + 8 * i4 + 4 * g < a.D) *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
       }
     if (g == 0) a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq] = (l > 0.f) ? m + log2f(l) : kNegInf;
   }

@@ -367,12 +367,21 @@ struct AsyncTileLoader {
   int row_in_pass;  // row of this lane within one pass over the tile
   int gchunk;       // logical chunk this lane fetches
   int wave;
+  // Byte offset of a lane whose chunk lies beyond the tensor's head dim (head dims below the tile width run
+  // zero-padded): past the end of every descriptor, so the range check fills the chunk with zeros.
+  static constexpr int kPadOffset = 0x7ffffff0;
 
-  __device__ __forceinline__ void init(int tid) {
+  // `d`: head dim of the tensors, a multiple of 8 not above HD
+  __device__ __forceinline__ void init(int tid, int d = HD) {
     const int lane = tid & 63;
     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     row_in_pass = wave * RPW + lane / CH;
     gchunk = (lane % CH) ^ Tile<HD>::swz(row_in_pass);
+    if (gchunk * 8 >= d) gchunk = -1;
+  }
+  // this lane's byte offset inside a tile whose rows are `stride_bytes` apart
+  __device__ __forceinline__ int lane_offset(int stride_bytes) const {
+    return gchunk < 0 ? kPadOffset : row_in_pass * stride_bytes + gchunk * 16;
   }
   // A source of rows: fixed descriptor over rows [row_base, row_end) of a (batch, head) slice whose
   // byte span fits 31 bits (kernels that may meet wider slices use load() below, which anchors a
@@ -391,7 +400,7 @@ struct AsyncTileLoader {
     const int64_t nbytes = (int64_t)(row_end > row_base ? row_end - row_base : 0) * s.stride_bytes;
     s.base = slice + (int64_t)row_base * row_stride;
     s.nbytes = nbytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)nbytes;
-    s.voff = row_in_pass * s.stride_bytes + gchunk * 16;
+    s.voff = lane_offset(s.stride_bytes);
     return s;
   }
   // rows [row0, row0 + ROWS) of the source into `tile`; rows past the source's end arrive as zeros
@@ -408,7 +417,7 @@ struct AsyncTileLoader {
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const uint32_t nbytes = rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
     const i32x4 rs = rsrc_words(src + (int64_t)row0 * row_stride, nbytes);
-    const int voff = row_in_pass * (int)stride_bytes + gchunk * 16;
+    const int voff = lane_offset((int)stride_bytes);
 #pragma unroll
     for (int i = 0; i < N; i++)
       lds_dma<16>(rs, lds_addr(tile + (i * NW + wave) * 512), voff, i * NW * RPW * (int)stride_bytes);

@@ -152,6 +152,13 @@ VARIANTS = [
     (1, 100, 2, 32, 3, 2, "chunk_visible", 8, torch.float32),
     (1, 100, 2, 96, 3, 2, "causal", 0, torch.bfloat16),
     (1, 60, 1, 256, 2, 1, "causal", 0, torch.float16),
+    # head dims below the matrix kernels' tile widths (64, 128): zero-padded inside the kernels
+    (2, 70, 2, 32, 3, 2, "causal", 0, torch.bfloat16),
+    (1, 150, 2, 96, 5, 4, "chunk_visible", 16, torch.float16),
+    (2, 64, 3, 96, 4, 1, "depth_only", 0, torch.bfloat16),
+    (1, 100, 2, 72, 2, 2, "noncausal", 0, torch.bfloat16),
+    (1, 90, 1, 8, 2, 2, "causal", 0, torch.float16),
+    (1, 200, 2, 120, 3, 4, "causal", 0, torch.bfloat16),
     (2, 45, 2, 36, 3, 2, "causal", 0, torch.bfloat16),     # rows of 72 bytes: not 16-byte aligned
     (1, 40, 3, 100, 2, 1, "noncausal", 0, torch.float16),  # rows of 200 bytes
 ]
@@ -712,6 +719,7 @@ def test_depth_gradients_accumulate_over_layers(gpu_device, case):
     (1, 1100, 2, 128, 0, 2, "causal", torch.float16),      # ragged last tile, two segments
     (1, 1024, 2, 128, 1, 2, "noncausal", torch.bfloat16),
     (1, 1024, 1, 128, 3, 4, "chunk_visible", torch.bfloat16),
+    (1, 1024, 1, 96, 1, 4, "causal", torch.bfloat16),      # padded head dim: the partial sums use the tile width
 ])
 def test_row_split_sequence_gradients(gpu_device, case):
     """Launches with few key tiles cut every tile's query rows into segments that leave fp32 partial sums for a
@@ -1021,6 +1029,8 @@ def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, variant):
     (64, 129, 8, 128, 2, 2, "chunk_visible", 16, torch.bfloat16),
     (64, 65, 8, 128, 7, 4, "depth_only", 0, torch.float16),
     (128, 257, 4, 64, 1, 1, "causal", 0, torch.bfloat16),
+    (32, 300, 16, 96, 3, 2, "causal", 0, torch.bfloat16),
+    (64, 130, 8, 32, 2, 1, "noncausal", 0, torch.float16),
 ], ids=lambda c: f"{c[6]}-B{c[0]}-T{c[1]}-D{c[3]}-L{c[4]}-G{c[5]}")
 def test_large_launch_shape_on_ragged_inputs(gpu_device, case):
     B, T, H, D, L, G, mode, cb, dtype = case
