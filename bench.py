@@ -34,6 +34,10 @@ WORKLOADS = {
     "c5": (64, 197, 6, 1, 64, 12, "noncausal", 0),
     "c5fda": (64, 197, 6, 1, 64, 12, "depth_only", 0),
     "plain": (1, 65536, 4, 4, 128, 0, "plain", 0),
+    # c2 with a head dim between the matrix kernels' tile widths (runs zero-padded to 128)
+    "c2d96": (2, 4096, 4, 4, 96, 8, "causal", 0),
+    # the last block of the reference's smallest MoDA vision model (4 query heads on 1 kv head, 11 earlier layers)
+    "deit_tiny": (64, 197, 1, 4, 64, 11, "noncausal", 0),
     "plain_c2": (2, 4096, 4, 4, 128, 0, "plain", 0),
     "plain_c3": (1, 16384, 4, 4, 128, 0, "plain", 0),
     # the c4 token count as one packed variable-length batch (cu_seqlens): 1 x 16K, 2 x 8K, 4 x 4K, 8 x 2K tokens
