@@ -261,7 +261,8 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # what FETCH_SIZE / WRITE_SIZE (KiB per dispatch) read for a plain copy of known size (the depth reorganisation
 # kernel of the same runs): FETCH_SIZE counts half of the bytes read, WRITE_SIZE all bytes written
 PMC_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
-KERNEL_NAMES = ("fwd_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "depth_cols_kernel", "reorg_kernel")
+KERNEL_NAMES = ("fwd_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "dkv_reduce_kernel", "depth_cols_kernel",
+                "chunk_depth_kernel", "reorg_kernel")
 
 
 def recorded_traffic(workload):
@@ -457,13 +458,17 @@ def main():
     traffic = recorded_traffic(args.workload) or {}
     # the dK/dV stage is timed as a whole: outside chunk-visible mode it is dkv_kernel followed by the HBM-bound
     # depth_cols_kernel
-    two_launches = dom == "dkv_kernel" and L > 0 and mode != "chunk_visible"
+    # (chunk-visible: dkv_kernel followed by chunk_depth_kernel; light launches add dkv_reduce_kernel)
+    two_launches = dom == "dkv_kernel" and L > 0
+    depth_kernel = "chunk_depth_kernel" if mode == "chunk_visible" else "depth_cols_kernel"
     dom_traffic = None
     if dom in traffic:
-        dom_traffic = traffic[dom]["bytes"] + (traffic.get("depth_cols_kernel", {}).get("bytes", 0.0) if two_launches else 0.0)
+        dom_traffic = traffic[dom]["bytes"]
+        if dom == "dkv_kernel":
+            dom_traffic += sum(traffic.get(k, {}).get("bytes", 0.0) for k in (depth_kernel, "dkv_reduce_kernel"))
     roofline = {
         "bound": "mfma",
-        "kernel": "dkv_kernel + depth_cols_kernel" if two_launches else dom,
+        "kernel": f"dkv_kernel + {depth_kernel}" if two_launches else dom,
         "achieved": kernels[dom]["tflops"],
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
@@ -475,7 +480,7 @@ def main():
     if hbm_bound(r["shape"], total_flops):
         mb = min_hbm_bytes(B, T, Hkv, G, D, L, mode)
         gbs = mb / (r["ms_step"] * 1e-3) / 1e9
-        whole = sum(v["bytes"] for v in traffic.values()) if traffic else None
+        whole = sum(v["bytes"] for k, v in traffic.items() if k != "reorg_kernel") if traffic else None
         roofline = {"bound": "hbm", "kernel": "fwd_kernel + delta_kernel + dq_kernel + dkv_kernel + depth_cols_kernel",
                     "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                     "algorithmic_bytes": mb, "traffic": whole,
