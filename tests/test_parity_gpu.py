@@ -490,10 +490,10 @@ def test_deit_style_caller_under_autocast(gpu_device):
 
 
 def test_integration_stub_as_documented(gpu_device, monkeypatch):
-    """INTEGRATION.md shows the ctypes binding a maintainer of the reference would put in place of the bodies of
-    parallel_moda_fwd / parallel_moda_bwd (moda_v14.py:381-522, 1470-1842).  This runs that very text (only
-    ctypes and torch; the library is found next to the package instead of on the loader path) and holds its
-    results to the parity bar."""
+    """The repository's integration notes show the ctypes binding a maintainer of the reference would put in place
+    of the bodies of parallel_moda_fwd / parallel_moda_bwd (moda_v14.py:381-522, 1470-1842).  This runs that very
+    text (only ctypes and torch; the library is found next to the package instead of on the loader path) and holds
+    its results to the parity bar."""
     import ctypes
     import os
     import re
@@ -507,7 +507,7 @@ def test_integration_stub_as_documented(gpu_device, monkeypatch):
     monkeypatch.setattr(ctypes, "CDLL", lambda name, *a, **kw: real_cdll(
         os.path.join(os.path.dirname(moda_amd.__file__), name) if name == "libmoda_hip.so" else name, *a, **kw))
     ns = {}
-    exec(compile(block, "INTEGRATION.md", "exec"), ns)
+    exec(compile(block, "integration-notes-stub", "exec"), ns)
     for (B, T, H, D, L, G, causal, dtype) in [(2, 150, 2, 64, 5, 2, True, torch.bfloat16),
                                               (1, 197, 3, 128, 4, 1, False, torch.float16),
                                               (1, 90, 2, 128, 0, 4, True, torch.bfloat16)]:
