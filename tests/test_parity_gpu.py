@@ -1140,6 +1140,55 @@ def test_random_sweep(gpu_device, seed):
     compare_all(got, ref, dtype, f"sweep {seed}")
 
 
+def _random_case_wide(seed):
+    """A second family: head dims below the tile widths, sequences long enough for the row split of the dK/dV
+    kernel, chunks above and below one query tile."""
+    import random
+
+    rnd = random.Random(seed)
+    mode = rnd.choice(["causal", "noncausal", "chunk_visible", "chunk_visible", "depth_only"])
+    D = rnd.choice([8, 32, 64, 72, 96, 128])
+    G = rnd.choice([1, 2, 4, 8, 16])
+    H = rnd.choice([1, 2])
+    L = rnd.choice([0, 1, 3, 6]) if mode != "depth_only" else rnd.choice([1, 3, 6])
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    T = rnd.choice([40, 129, 300, 520, 700, 1100])
+    if mode == "depth_only":
+        T = min(T, 520)
+    T = min(T, 4400 // G)  # keeps the dense oracle's score matrix small
+    B = rnd.choice([1, 2]) if T * G <= 2400 else 1
+    cb = rnd.choice([1, 4, 16, max(1, 64 // G), max(1, 128 // G), 40]) if mode == "chunk_visible" else 0
+    valid = None
+    if L > 1 and mode != "chunk_visible" and rnd.random() < 0.3:
+        valid = rnd.randint(1, L)
+    return mode, D, G, H, L, dtype, T, B, cb, valid
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_sweep_wide(gpu_device, seed):
+    from moda_amd import ops
+
+    mode, D, G, H, L, dtype, T, B, cb, valid = _random_case_wide(5000 + seed)
+    say(f"[wide sweep {seed}] mode={mode} D={D} G={G} H={H} L={L} {dtype} T={T} B={B} cb={cb} valid={valid}")
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=seed, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
+    sc = D ** -0.5
+    ref_inp = dict(inp)
+    if valid is not None:
+        ref_inp["kd"] = oracle.compact_depth(inp["kd"], T, valid)
+        ref_inp["vd"] = oracle.compact_depth(inp["vd"], T, valid)
+    ref = oracle.moda_dense_fwd_bwd(ref_inp, sc, G, mode, cb)
+    if valid is not None:
+        ref["dkd"] = oracle.scatter_depth_grad(ref["dkd"], T, L)
+        ref["dvd"] = oracle.scatter_depth_grad(ref["dvd"], T, L)
+    dev = to_dev(inp, gpu_device)
+    m = MODE_ID[mode]
+    o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], sc, G, cb, depth_valid=valid)
+    dq, dk, dv, dkd, dvd = ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], o, lse, dev["do"], sc, G,
+                                        cb, depth_valid=valid)
+    got = {"o": o, "lse": lse, "dq": dq, "dk": dk, "dv": dv, "dkd": dkd, "dvd": dvd}
+    compare_all(got, ref, dtype, f"wide sweep {seed}")
+
+
 def test_more_than_65535_batch_heads(gpu_device):
     """Launch grids are one-dimensional: batch x heads beyond the 65535 limit of a grid's y extent."""
     B, T, H, D, L, G = 70000, 3, 1, 64, 2, 2
