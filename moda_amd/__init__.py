@@ -21,6 +21,8 @@ from .ops import (  # noqa: F401
     ParallelMixtureOfDepthAttentionChunkVisibleFunction,
     ParallelFlashDepthAttentionFunction,
     ParallelAttentionFunction,
+    fold_gqa_heads,
+    unfold_gqa_heads,
 )
 from .depth_cache import build_depth_cache, stack_depth, DepthCache  # noqa: F401
 from .modules import DepthStream, MoDAAttention, MoDAStack  # noqa: F401
@@ -38,6 +40,8 @@ __all__ = [
     "parallel_attn",
     "parallel_attn_fwd",
     "parallel_attn_bwd",
+    "fold_gqa_heads",
+    "unfold_gqa_heads",
     "build_depth_cache",
     "stack_depth",
     "DepthCache",

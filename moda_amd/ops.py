@@ -634,6 +634,39 @@ def parallel_fda(q, k=None, v=None, g=None, cached_k=None, cached_v=None, scale=
 
 
 # ---------------------------------------------------------------------------
+# head-dim GQA <-> the folded layout of the depth modes
+# ---------------------------------------------------------------------------
+def fold_gqa_heads(x: torch.Tensor, num_kv_heads: int, head_order: str = "group_major") -> torch.Tensor:
+    """``[B, T, Hq, D]`` (one query head per head-dim slot) -> the folded ``[B, T*G, Hkv, D]`` that
+    ``parallel_moda`` / ``parallel_moda_chunk_visible`` / ``parallel_fda`` take with ``moda_group_num = G``,
+    ``G = Hq // Hkv``: the G query heads that share a kv head become G consecutive rows of the token.
+
+    Which query heads share a kv head is a convention of the model, so it is an explicit argument:
+    ``"group_major"`` -- query head ``g*Hkv + hkv`` reads kv head ``hkv`` (the fold of the reference's vision
+    model, vision_tasks/deit/models.py:248-250); a free view of a contiguous ``x``.
+    ``"kv_major"`` -- query head ``hkv*G + g`` reads kv head ``hkv`` (``repeat_interleave`` models and the plain
+    comparator, fla/ops/attn/parallel.py:48-49); needs one copy."""
+    B, T, Hq, D = x.shape
+    assert Hq % num_kv_heads == 0, "query heads must be a multiple of kv heads"
+    G = Hq // num_kv_heads
+    if head_order == "group_major":
+        return x.reshape(B, T, G, num_kv_heads, D).reshape(B, T * G, num_kv_heads, D)
+    assert head_order == "kv_major", "head_order must be 'group_major' or 'kv_major'"
+    return x.reshape(B, T, num_kv_heads, G, D).transpose(2, 3).reshape(B, T * G, num_kv_heads, D)
+
+
+def unfold_gqa_heads(x: torch.Tensor, moda_group_num: int, head_order: str = "group_major") -> torch.Tensor:
+    """Inverse of :func:`fold_gqa_heads`: ``[B, T*G, Hkv, D]`` -> ``[B, T, G*Hkv, D]``."""
+    B, TG, Hkv, D = x.shape
+    G = moda_group_num
+    assert TG % G == 0, "rows must be a multiple of moda_group_num"
+    if head_order == "group_major":
+        return x.reshape(B, TG // G, G * Hkv, D)
+    assert head_order == "kv_major", "head_order must be 'group_major' or 'kv_major'"
+    return x.reshape(B, TG // G, G, Hkv, D).transpose(2, 3).reshape(B, TG // G, Hkv * G, D)
+
+
+# ---------------------------------------------------------------------------
 # plain causal attention with head-dim GQA -- fla/ops/attn/parallel.py
 # ---------------------------------------------------------------------------
 def parallel_attn_fwd(q, k, v, g_cumsum=None, scale=None, cu_seqlens=None):

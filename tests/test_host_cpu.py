@@ -219,6 +219,35 @@ def test_depth_cache_append_checks_the_layer_against_the_cache():
         moda_amd.depth_cache._reorg_fwd([z(2, 8, 2, 64)], z(2, 16, 2, 64), 0, 3)
 
 
+def test_gqa_head_folds_match_the_two_head_conventions():
+    """fold_gqa_heads turns head-dim GQA queries into the folded layout of the depth modes.  Pinned on the oracle:
+    kv_major folding + the folded operator == the plain comparator (query head hq reads kv head hq // G, the
+    repeat_interleave convention); group_major folding == the reference caller's reshape; both invert exactly."""
+    import moda_amd
+    import oracle
+
+    gen = torch.Generator().manual_seed(3)
+    B, T, Hkv, G, D = 2, 9, 2, 3, 8
+    q = torch.randn(B, T, Hkv * G, D, generator=gen, dtype=torch.float64)
+    k = torch.randn(B, T, Hkv, D, generator=gen, dtype=torch.float64)
+    v = torch.randn(B, T, Hkv, D, generator=gen, dtype=torch.float64)
+    ref, _ = oracle.plain_gqa_dense(q, k, v, dtype=torch.float64)
+    qf = moda_amd.fold_gqa_heads(q, Hkv, "kv_major")
+    o, _ = oracle.moda_dense(qf, k, v, None, None, None, G, "causal", dtype=torch.float64)
+    assert torch.allclose(moda_amd.unfold_gqa_heads(o, G, "kv_major"), ref, atol=1e-12)
+    # group-major: query head g*Hkv + hkv reads kv head hkv, i.e. the caller's q.reshape(B, N, G, Hkv, D)
+    qg = moda_amd.fold_gqa_heads(q, Hkv, "group_major")
+    assert torch.equal(qg, q.reshape(B, T, G, Hkv, D).reshape(B, T * G, Hkv, D))
+    assert qg.data_ptr() == q.data_ptr()  # a view, no copy
+    o, _ = oracle.moda_dense(qg, k, v, None, None, None, G, "causal", dtype=torch.float64)
+    kk = torch.cat([k] * G, dim=2)  # kv head of query head g*Hkv + hkv is hkv
+    vv = torch.cat([v] * G, dim=2)
+    ref_g, _ = oracle.plain_gqa_dense(q, kk, vv, dtype=torch.float64)  # one kv head per query head
+    assert torch.allclose(moda_amd.unfold_gqa_heads(o, G, "group_major"), ref_g, atol=1e-12)
+    for order in ("group_major", "kv_major"):
+        assert torch.equal(moda_amd.unfold_gqa_heads(moda_amd.fold_gqa_heads(q, Hkv, order), G, order), q)
+
+
 def test_compat_package_reexports():
     import sys
 
