@@ -3,8 +3,10 @@
 // fda_v12.py:646-860, fla/ops/attn/parallel.py:299-440).
 //
 // A workgroup (eight waves) owns 128 key columns of one (batch, kv head) --
-// sequence keys or flattened depth slots -- as four 32-column blocks, one column
-// per lane pair.  It streams 64-row query tiles (Q, dO, LSE, delta) through a
+// sequence keys or flattened depth slots -- as four 32-column blocks; the products
+// run on the 16x16x32 matrix instruction (less power per multiply-add than 32x32x16
+// on a power-limited matrix pipe), a block being two 16-column halves with lane
+// (n, q) on columns 16*nb + n.  It streams 64-row query tiles (Q, dO, LSE, delta) through a
 // three-stage LDS ring (one tile in flight while each role consumes one), from
 // the last tile down to its
 // diagonal (workgroups that run together then read the same tiles at the same
@@ -23,6 +25,7 @@
 
 #include "kargs.h"
 #include "tile.h"
+#include "tile16.h"
 
 namespace moda {
 
@@ -31,7 +34,7 @@ namespace moda {
 template <typename T, int HD, bool VARLEN, bool SPLIT = false>
 __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   static_assert(!(VARLEN && SPLIT), "packed batches are not split");
-  constexpr int BN = 128, BM = 64, KK = HD / 16, DB = HD / 32, NST = 3;
+  constexpr int BN = 128, BM = 64, KS = HD / 32, MB = HD / 16, NST = 3;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
   // ring of NST stages, each: Q tile, dO tile; then the P mailbox; then lse/delta per stage
@@ -39,7 +42,8 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   MODA_LDS i32x4* mbox = (MODA_LDS i32x4*)(smem + NST * 2 * BM * HD);      // [2 parities][4 blocks][4][64 lanes]
   MODA_LDS float* stat = (MODA_LDS float*)(mbox + 2 * 4 * 4 * 64);         // [NST][2][BM]
 
-  const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+  // lane (n, q4) owns columns 16*nb + n (nb = 0, 1) of the wave's block
+  const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kblk = wave & 3;
   const bool role_b = wave >= 4;
@@ -67,24 +71,31 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   }
   const int c_first = tile * BN;
   if (VARLEN && c_first >= ncols) return;  // a tile beyond this sequence of a variable-length batch
-  const int c = c_first + kblk * 32 + n;
-  const bool valid = c < ncols;
-  // a depth slot without data: no row sees it; its K/V are replaced by zeros, its gradients come out zero
-  const bool empty_slot = dep && valid && (c % a.L) >= a.Lv;
+  int c[2];
+  bool valid[2], live[2];  // live: a column with data (an unwritten depth slot is seen by no row: its K/V are
+                           // replaced by zeros, its gradients come out zero)
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++) {
+    c[nb] = c_first + kblk * 32 + 16 * nb + n;
+    valid[nb] = c[nb] < ncols;
+    live[nb] = valid[nb] && !(dep && (c[nb] % a.L) >= a.Lv);
+  }
 
   // stationary operand of this wave's role: K rows (A) or V rows (B)
-  i32x4 Sr[KK];
+  i32x4 Sr[2][KS];
   {
     const uint16_t* src = role_b ? (dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h)
                                  : (dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h);
     const int64_t st = role_b ? (dep ? a.svd.t : a.sv.t) : (dep ? a.skd.t : a.sk.t);
 #pragma unroll
-    for (int kk = 0; kk < KK; kk++) {
-      i32x4 z = {0, 0, 0, 0};
-      Sr[kk] = (valid && !empty_slot && 16 * kk + 8 * g < a.D)
-                   ? *reinterpret_cast<const i32x4*>(src + (int64_t)c * st + 16 * kk + 8 * g)
-                   : z;
-    }
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        i32x4 z = {0, 0, 0, 0};
+        Sr[nb][ks] = (live[nb] && 32 * ks + 8 * q4 < a.D)
+                         ? *reinterpret_cast<const i32x4*>(src + (int64_t)c[nb] * st + 32 * ks + 8 * q4)
+                         : z;
+      }
   }
 
   // The register operands above must have arrived before the tile loads start: those are issued
@@ -105,8 +116,10 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
       hi = a.chunk ? min(a.T, (w / a.Cb + 1) * a.Cb) * a.Gf : (w + 1) * a.Gf;
     }
   };
-  int qlo = 0, qhi = 0;
-  if (valid && !empty_slot) q_interval(c, qlo, qhi);
+  int qlo[2] = {0, 0}, qhi[2] = {0, 0};
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++)
+    if (live[nb]) q_interval(c[nb], qlo[nb], qhi[nb]);
   int wg_lo, wg_hi, tmp;
   q_interval(c_first, wg_lo, tmp);
   q_interval(min(ncols, c_first + BN) - 1, tmp, wg_hi);
@@ -187,13 +200,13 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
     if (j % every == 1 && j / every < kParts) part(j / every);
   };
 
-  f32x16 acc[DB];  // dV^T (role A) or dK^T (role B)
+  f32x4 acc[MB][2];  // dV^T (role A) or dK^T (role B): head-dim block x column block
 #pragma unroll
-  for (int d = 0; d < DB; d++)
+  for (int d = 0; d < MB; d++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) acc[d][i] = 0.f;
+    for (int nb = 0; nb < 2; nb++) acc[d][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float sc = a.scale * kLog2e;
-  OperandAddr<HD> oa;
+  Operand16<HD> oa;
   oa.init(lane);
 
   feeding = niter > 0;
@@ -219,62 +232,66 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
 
   // role A, one tile: S = Q K^T, P = exp2(S c - lse) -> mailbox, dV^T += dO^T P
   auto tile_a = [&](bool masked, lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* lse_s, MODA_LDS i32x4* mb, int q0) {
-    f32x16 s[2];
-    mfma_rows<T, HD, 2, 4>(oa, Qs, Sr, s, feed);
-    TrPipe<T, HD, 4, 2> dvp;
+    f32x4 s[4][2];
+    mfma16_rows<T, HD, 4, 2, 4>(oa, Qs, Sr, s, feed);
+    TrPipe16<T, HD, 2, 2, 2> dvp;
     dvp.prefetch(oa, dOs);
 #pragma unroll
-    for (int bb = 0; bb < 2; bb++)
+    for (int m = 0; m < 4; m++) {
+      const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + 16 * m + slot_base(q4));
 #pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + 32 * bb + 8 * i4 + 4 * g);
+      for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) s[bb][4 * i4 + j] = fast_exp2(__builtin_fmaf(s[bb][4 * i4 + j], sc, -lv[j]));
-      }
+        for (int j = 0; j < 4; j++) s[m][nb][j] = fast_exp2(__builtin_fmaf(s[m][nb][j], sc, -lv[j]));
+    }
     if (masked) {  // wave-uniform; touches only s, so the accumulators stay where they are
 #pragma unroll
-      for (int bb = 0; bb < 2; bb++)
+      for (int m = 0; m < 4; m++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const int qr = q0 + 32 * bb + 8 * (i >> 2) + 4 * g + (i & 3);
-          s[bb][i] = (qr >= qlo && qr < qhi) ? s[bb][i] : 0.f;
-        }
-    }
-    i32x4 P[4];
+        for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
-      mb[ks * 64] = P[ks];
+          for (int j = 0; j < 4; j++) {
+            const int qr = q0 + 16 * m + slot_base(q4) + j;
+            s[m][nb][j] = (qr >= qlo[nb] && qr < qhi[nb]) ? s[m][nb][j] : 0.f;
+          }
     }
+    i32x4 P[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) {
+        P[ks][nb] = pack_slots<T>(s[2 * ks][nb], s[2 * ks + 1][nb]);
+        mb[(2 * ks + nb) * 64] = P[ks][nb];
+      }
     dvp.run(oa, dOs, P, acc);
   };
   // role B, one tile: dP - delta = dO V^T with the accumulators preset to -delta (the workspace holds
   // minus delta), dS = P (dP - delta), dK^T += Q^T dS
   auto tile_b = [&](lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* del_s, MODA_LDS const i32x4* mb) {
-    f32x16 dp[2];
+    f32x4 dp[4][2];
 #pragma unroll
-    for (int bb = 0; bb < 2; bb++)
-#pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const f32x4 dv = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + 32 * bb + 8 * i4 + 4 * g);
-#pragma unroll
-        for (int j = 0; j < 4; j++) dp[bb][4 * i4 + j] = dv[j];
-      }
-    mfma_rows_acc<T, HD, 2, 4>(oa, dOs, Sr, dp, feed);
-    TrPipe<T, HD, 4, 2> dkp;
-    dkp.prefetch(oa, Qs);
-    i32x4 DS[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      const int bb = ks >> 1;
-      const i32x4 pw = mb[ks * 64];
-      float p[8];
-#pragma unroll
-      for (int w = 0; w < 4; w++) unpack2<T>(pw[w], p[2 * w], p[2 * w + 1]);
-#pragma unroll
-      for (int w = 0; w < 4; w++)
-        DS[ks][w] = pack2<T>(p[2 * w] * dp[bb][8 * (ks & 1) + 2 * w], p[2 * w + 1] * dp[bb][8 * (ks & 1) + 2 * w + 1]);
+    for (int m = 0; m < 4; m++) {
+      const f32x4 dv = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + 16 * m + slot_base(q4));
+      dp[m][0] = dv;
+      dp[m][1] = dv;
     }
+    mfma16_rows<T, HD, 4, 2, 4, true>(oa, dOs, Sr, dp, feed);
+    TrPipe16<T, HD, 2, 2, 2> dkp;
+    dkp.prefetch(oa, Qs);
+    i32x4 DS[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) {
+        const i32x4 pw = mb[(2 * ks + nb) * 64];
+        float p[8];
+#pragma unroll
+        for (int w = 0; w < 4; w++) unpack2<T>(pw[w], p[2 * w], p[2 * w + 1]);
+        DS[ks][nb][0] = pack2<T>(p[0] * dp[2 * ks][nb][0], p[1] * dp[2 * ks][nb][1]);
+        DS[ks][nb][1] = pack2<T>(p[2] * dp[2 * ks][nb][2], p[3] * dp[2 * ks][nb][3]);
+        DS[ks][nb][2] = pack2<T>(p[4] * dp[2 * ks + 1][nb][0], p[5] * dp[2 * ks + 1][nb][1]);
+        DS[ks][nb][3] = pack2<T>(p[6] * dp[2 * ks + 1][nb][2], p[7] * dp[2 * ks + 1][nb][3]);
+      }
     dkp.run(oa, Qs, DS, acc);
   };
 
@@ -314,7 +331,8 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
       MODA_LDS const float* st_s = stat + st * 2 * BM;
       bool run = true;
       if (MASKED) {
-        run = __any((qhi > q0) && (qlo < q0 + BM) && (qhi > qlo));
+        run = __any(((qhi[0] > q0) && (qlo[0] < q0 + BM) && (qhi[0] > qlo[0])) ||
+                    ((qhi[1] > q0) && (qlo[1] < q0 + BM) && (qhi[1] > qlo[1])));
         if (!run) {
 #pragma unroll
           for (int k = 0; k < kParts; k++) part(k);
@@ -362,45 +380,40 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
 
   if (SPLIT && !dep) {
     // a row segment: fp32 partial sums, added up by dkv_reduce_kernel
-    if (valid) {
-      const int64_t plane = (int64_t)a.B * a.Hkv * a.T * HD;
-      float* outp = a.dkv_part + ((int64_t)(role_b ? 0 : 1) * nseg + seg) * plane +
-                    (((int64_t)b * a.Hkv + hkv) * a.T + c) * HD;
-      const float mul = role_b ? a.scale : 1.f;
+    const int64_t plane = (int64_t)a.B * a.Hkv * a.T * HD;
+    const float mul = role_b ? a.scale : 1.f;
 #pragma unroll
-      for (int d = 0; d < DB; d++)
+    for (int nb = 0; nb < 2; nb++)
+      if (valid[nb]) {
+        float* outp = a.dkv_part + ((int64_t)(role_b ? 0 : 1) * nseg + seg) * plane +
+                      (((int64_t)b * a.Hkv + hkv) * a.T + c[nb]) * HD;
 #pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          f32x4 w;
-#pragma unroll
-          for (int j = 0; j < 4; j++) w[j] = acc[d][4 * i4 + j] * mul;
-          *reinterpret_cast<f32x4*>(outp + 32 * d + 8 * i4 + 4 * g) = w;
-        }
-    }
+        for (int d = 0; d < MB; d++) *reinterpret_cast<f32x4*>(outp + 16 * d + 4 * q4) = acc[d][nb] * mul;
+      }
     return;
   }
-  if (valid) {
-    uint16_t* outp;
-    float mul;
-    if (!role_b) {  // dV
-      outp = dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)c * a.sdvd.t
-                 : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t;
-      mul = 1.f;
-    } else {  // dK
-      outp = dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)c * a.sdkd.t
-                 : a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t;
-      mul = a.scale;
-    }
 #pragma unroll
-    for (int d = 0; d < DB; d++)
-#pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        i32x2 w;
-        w[0] = pack2<T>(acc[d][4 * i4 + 0] * mul, acc[d][4 * i4 + 1] * mul);
-        w[1] = pack2<T>(acc[d][4 * i4 + 2] * mul, acc[d][4 * i4 + 3] * mul);
-        if (32 * d + 8 * i4 + 4 * g < a.D) *reinterpret_cast<i32x2*>(outp + 32 * d + 8 * i4 + 4 * g) = w;
+  for (int nb = 0; nb < 2; nb++)
+    if (valid[nb]) {
+      uint16_t* outp;
+      float mul;
+      if (!role_b) {  // dV
+        outp = dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)c[nb] * a.sdvd.t
+                   : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c[nb] * a.sdv.t;
+        mul = 1.f;
+      } else {  // dK
+        outp = dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)c[nb] * a.sdkd.t
+                   : a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c[nb] * a.sdk.t;
+        mul = a.scale;
       }
-  }
+#pragma unroll
+      for (int d = 0; d < MB; d++) {
+        i32x2 w;
+        w[0] = pack2<T>(acc[d][nb][0] * mul, acc[d][nb][1] * mul);
+        w[1] = pack2<T>(acc[d][nb][2] * mul, acc[d][nb][3] * mul);
+        if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(outp + 16 * d + 4 * q4) = w;
+      }
+    }
 }
 
 // Depth columns in chunk-visible mode when a chunk's query rows fit one 64-row tile (the reference's only

@@ -2,17 +2,21 @@
 // dQ kernel (moda_v14.py:542-871, moda_v16.py:936-1220, fda_v12.py:432-638,
 // fla/ops/attn/parallel.py:165-296).
 //
-// Same decomposition as the forward kernel: a workgroup owns 32 query rows per wave
-// (256 in the throughput launch shape, 64 or 128 in the small one),
-// one row per lane pair, and streams 64-column K/V tiles (sequence keys, then
-// the rows' depth slots).  P^T is recomputed from the saved base-2 LSE,
-// dS^T = P^T * (dP^T - delta) is packed straight into the B operand of
-// dQ^T += K^T * dS^T, K^T coming from the LDS transpose read of the K tile.
+// Same streaming structure as the forward kernel: a workgroup owns 32 query rows per wave
+// (256 in the throughput launch shape, 64 or 128 in the small one) and streams 64-column K/V tiles
+// (sequence keys, then the rows' depth slots) through an LDS ring.  The products run on the 16x16x32
+// matrix instruction, which moves a quarter of the accumulator bits per multiply-add of the 32x32x16
+// one and draws less power on a matrix pipe whose clock the power limit sets (measured on the
+// long-sequence workload: about 9 % less time for the same tiles).  A wave's 32 rows are two 16-row
+// blocks; lane (n, q) owns rows 16*nb + n and, inside a 16-column score block, columns slot_base(q) .. +3.
+// P^T is recomputed from the saved base-2 LSE, dS^T = P^T * (dP^T - delta) is packed straight into the
+// B operand of dQ^T += K^T * dS^T, K^T coming from the LDS transpose read of the K tile.
 #include <algorithm>
 #include <type_traits>
 
 #include "kargs.h"
 #include "tile.h"
+#include "tile16.h"
 #include "tuning.h"
 
 namespace moda {
@@ -50,13 +54,12 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a_in) {
 // offsets inside the slice); bit 1: packed variable-length batch
 template <typename T, int HD, typename Shape, int ADDR>
 __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) {
-  constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST, DIST = Shape::DIST;
+  constexpr int BM = 32 * Shape::W, BN = 64, KS = HD / 32, MB = HD / 16, NT = 64 * Shape::W, NST = Shape::NST, DIST = Shape::DIST;
   static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
-  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, q4 = lane >> 4;
   constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0;
   const int BH = a_in.B * a_in.Hq;
   const int bh = blockIdx.x % BH;
@@ -65,57 +68,51 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   SeqArgs<VARLEN> seq(a_in, b);
   const KArgs& a = seq.a;
   const int nqt = (a.Tq + BM - 1) / BM;
-  // Heavy (late) tiles first.  In a variable-length batch the grid counts tiles from the end of the longest
-  // sequence, so that tiles of equal cost (equal row position) of all sequences are dispatched together and the
-  // heaviest of the whole batch first; the positions a shorter sequence does not have are dropped.
   const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
   if (VARLEN && qt >= nqt) return;
-  const int r = qt * BM + wave * 32 + n;
-  const bool valid = r < a.Tq;
-  const int t = r / a.Gf;
 
-  i32x4 Qr[KK], dOr[KK];
-  float lse = 0.f, delta = 0.f;
-  {
-    const uint16_t* qp = a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + 8 * g;
-    const uint16_t* dop = a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + 8 * g;
+  i32x4 Qr[2][KS], dOr[2][KS];
+  float lse[2], delta[2];
+  int shi[2], dlo[2], dhi[2];
 #pragma unroll
-    for (int kk = 0; kk < KK; kk++) {
+  for (int nb = 0; nb < 2; nb++) {
+    const int r = qt * BM + wave * 32 + 16 * nb + n;
+    const bool valid = r < a.Tq;
+    const uint16_t* qp = a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + 8 * q4;
+    const uint16_t* dop = a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + 8 * q4;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
       i32x4 z = {0, 0, 0, 0};
-      const bool in = valid && 16 * kk + 8 * g < a.D;
-      Qr[kk] = in ? *reinterpret_cast<const i32x4*>(qp + 16 * kk) : z;
-      dOr[kk] = in ? *reinterpret_cast<const i32x4*>(dop + 16 * kk) : z;
+      const bool in = valid && 32 * ks + 8 * q4 < a.D;
+      Qr[nb][ks] = in ? *reinterpret_cast<const i32x4*>(qp + 32 * ks) : z;
+      dOr[nb][ks] = in ? *reinterpret_cast<const i32x4*>(dop + 32 * ks) : z;
     }
+    lse[nb] = 0.f;
+    delta[nb] = 0.f;
+    shi[nb] = dlo[nb] = dhi[nb] = 0;
     if (valid) {
-      lse = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq];
-      delta = a.delta[((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r];
+      lse[nb] = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq];
+      delta[nb] = a.delta[((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r];
+      const int t = r / a.Gf;
+      if (a.has_seq) shi[nb] = a.causal ? t + 1 : a.T;
+      if (a.L > 0) {
+        const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
+        dlo[nb] = lo_t * a.L;
+        dhi[nb] = a.chunk ? (t + 1) * a.L : dlo[nb] + a.Lv;
+      }
     }
   }
-
-  // The register operands above must have arrived before the tile loads start: those are issued
-  // behind the compiler's back, and a load it still believes pending would cost a vmcnt(0) in every
-  // trip of the main loop.
-  asm volatile("" ::: "memory");  // keep the loads above this point
+  // the register operands must have arrived before the tile loads (issued behind the compiler's back) start
+  asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt(0x0F70);
   asm volatile("" ::: "memory");
 
-  int shi = 0, dlo = 0, dhi = 0;
-  if (valid) {
-    if (a.has_seq) shi = a.causal ? t + 1 : a.T;
-    if (a.L > 0) {
-      const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
-      dlo = lo_t * a.L;
-      dhi = a.chunk ? (t + 1) * a.L : dlo + a.Lv;  // the token's filled slots
-    }
-  }
   const int r_first = qt * BM;
   const int r_last = min(a.Tq, r_first + BM) - 1;
   const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
   int n_seq = 0, n_full = 0;
   if (a.has_seq) {
     n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
-    // leading sequence tiles every row of the workgroup sees completely (padding rows of the last
-    // workgroup carry zero queries and zero dO there and are never stored)
     n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
   }
   int dep0 = 0, n_dep = 0;
@@ -124,25 +121,21 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     dep0 = lo_t * a.L;
     n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
   }
-  // wave-uniform by construction, but computed with vector divisions: the explicit hint keeps the
-  // loop control in scalar registers
   n_seq = __builtin_amdgcn_readfirstlane(n_seq);
   n_full = __builtin_amdgcn_readfirstlane(n_full);
   dep0 = __builtin_amdgcn_readfirstlane(dep0);
   const int ntiles = __builtin_amdgcn_readfirstlane(n_seq + n_dep);
 
   typedef AsyncTileLoader<HD, BN, NT> Loader;
-  constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
+  constexpr int LPT = 2 * Loader::N;
   Loader ld;
   ld.init(tid, a.D);
-  // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
-  // producer reaches the first depth tile
   typename Loader::Source srcK, srcV;
   if (a.has_seq && n_seq > 0) {
     srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
     srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
   }
-  int ld_st = 0;  // ring stage the next issued tile goes to
+  int ld_st = 0;
   auto issue = [&](int it) {
     lds_ptr Kt = smem + ld_st * 2 * BN * HD;
     if (it == n_seq) {
@@ -150,7 +143,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
       srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
-    if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
+    if (WIDE) {
       const bool dep = it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
@@ -163,7 +156,6 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     }
     ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
   };
-  // wait until tile `next` has landed; tiles next+1 .. next+DIST-1 may still be in flight
   auto wait_tile = [&](int next) {
     if (DIST == 2 && next + 1 < ntiles)
       Loader::template wait_but<LPT>();
@@ -171,13 +163,13 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
       Loader::wait_all();
   };
 
-  f32x16 dq[DB];
+  f32x4 dq[MB][2];
 #pragma unroll
-  for (int d = 0; d < DB; d++)
+  for (int d = 0; d < MB; d++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) dq[d][i] = 0.f;
+    for (int nb = 0; nb < 2; nb++) dq[d][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float sc = a.scale * kLog2e;
-  OperandAddr<HD> oa;
+  Operand16<HD> oa;
   oa.init(lane);
 
 #pragma unroll
@@ -185,57 +177,60 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     if (j < ntiles) issue(j);
   wait_tile(0);
   __syncthreads();
-  int c_st = 0;  // ring stage of the tile being consumed
+  int c_st = 0;
 
-  // start value of every dP^T accumulator block: this lane's row constant -rowsum(o * do), so that the
-  // subtraction costs no instruction per element
-  f32x16 dp_init;
+  f32x4 dp_init[2];
 #pragma unroll
-  for (int i = 0; i < 16; i++) dp_init[i] = delta;
-  // one column tile: S^T = K Q^T and dP^T = V dO^T in one MFMA pipeline, dS^T, dQ^T += K^T dS^T
-  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, int lo, int hi) {
+  for (int nb = 0; nb < 2; nb++) dp_init[nb] = f32x4{delta[nb], delta[nb], delta[nb], delta[nb]};
+  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, const int (&lo)[2], const int (&hi)[2]) {
     constexpr bool MASKED = decltype(masked)::value;
-    f32x16 s[2], dp[2];
-    mfma_rows2<T, HD, 2, 4>(oa, Kc, Qr, s, Vc, dOr, dp, dp_init);
-    TrPipe<T, HD, 4, 2> kt;
+    f32x4 s[4][2], dp[4][2];
+    mfma16_rows2<T, HD, 4, 2, 2>(oa, Kc, Qr, s, Vc, dOr, dp, dp_init);
+    TrPipe16<T, HD, 2, 2, 3> kt;
     kt.prefetch(oa, Kc);
 #pragma unroll
-    for (int bb = 0; bb < 2; bb++)
+    for (int mb = 0; mb < 4; mb++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, -lse));
-        if (MASKED) {
-          const int c = col0 + 32 * bb + acc_row(i, g);
-          p = (c >= lo && c < hi) ? p : 0.f;
+      for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float p = fast_exp2(__builtin_fmaf(s[mb][nb][i], sc, -lse[nb]));
+          if (MASKED) {
+            const int c = col0 + 16 * mb + slot_base(q4) + i;
+            p = (c >= lo[nb] && c < hi[nb]) ? p : 0.f;
+          }
+          s[mb][nb][i] = p * dp[mb][nb][i];
         }
-        s[bb][i] = p * dp[bb][i];  // dp started from minus rowsum(o * do)
-      }
-    i32x4 DS[4];
+    i32x4 DS[2][2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) DS[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) DS[ks][nb] = pack_slots<T>(s[2 * ks][nb], s[2 * ks + 1][nb]);
     kt.run(oa, Kc, DS, dq);
   };
 
-  // phase 1: tiles fully visible to every row -- no masks, no visibility tests.  (Not unrolled over the
-  // ring stages like the forward loop: this kernel has no registers left for a second set of operand
-  // addresses.)
   int it = 0;
+  const int none[2] = {0, 0};
   for (; it < n_full; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     lds_cptr Kc = smem + c_st * 2 * BN * HD;
-    tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, 0, 0);
+    tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, none, none);
     c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
     wait_tile(it + 1);
     __syncthreads();
   }
-  // phase 2: boundary sequence tiles and depth tiles
   for (; it < ntiles; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     const bool dep = it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
-    const int lo = dep ? dlo : 0;
-    const int hi = dep ? dhi : shi;
-    const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
+    int lo[2], hi[2];
+    bool touches = false;
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      lo[nb] = dep ? dlo[nb] : 0;
+      hi[nb] = dep ? dhi[nb] : shi[nb];
+      touches = touches || ((hi[nb] > col0) && (lo[nb] < col0 + BN) && (hi[nb] > lo[nb]));
+    }
     if (__any(touches)) {
       lds_cptr Kc = smem + c_st * 2 * BN * HD;
       tile(std::true_type{}, Kc, Kc + BN * HD, col0, lo, hi);
@@ -245,17 +240,19 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     __syncthreads();
   }
 
-  if (valid) {
-    uint16_t* op = a.dq + b * a.sdq.b + hq * a.sdq.h + (int64_t)r * a.sdq.t;
 #pragma unroll
-    for (int d = 0; d < DB; d++)
+  for (int nb = 0; nb < 2; nb++) {
+    const int r = qt * BM + wave * 32 + 16 * nb + n;
+    if (r < a.Tq) {
+      uint16_t* op = a.dq + b * a.sdq.b + hq * a.sdq.h + (int64_t)r * a.sdq.t;
 #pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
+      for (int d = 0; d < MB; d++) {
         i32x2 w;
-        w[0] = pack2<T>(dq[d][4 * i4 + 0] * a.scale, dq[d][4 * i4 + 1] * a.scale);
-        w[1] = pack2<T>(dq[d][4 * i4 + 2] * a.scale, dq[d][4 * i4 + 3] * a.scale);
-        if (32 * d + 8 * i4 + 4 * g < a.D) *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
+        w[0] = pack2<T>(dq[d][nb][0] * a.scale, dq[d][nb][1] * a.scale);
+        w[1] = pack2<T>(dq[d][nb][2] * a.scale, dq[d][nb][3] * a.scale);
+        if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(op + 16 * d + 4 * q4) = w;
       }
+    }
   }
 }
 

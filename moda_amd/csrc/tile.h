@@ -229,38 +229,6 @@ __device__ __forceinline__ void mfma_rows_acc(const OperandAddr<HD>& oa, lds_cpt
   }
 }
 
-// Two tiles against two register operands in one pipeline:
-// acc0[bb] = rows(tile0) x breg0, acc1[bb] = init1 + rows(tile1) x breg1 (init1: the same start value for every block).
-template <typename T, int HD, int NB, int DEPTH, typename Hook = NoHook>
-__device__ __forceinline__ void mfma_rows2(const OperandAddr<HD>& oa, lds_cptr tile0, const i32x4 (&breg0)[HD / 16],
-                                           f32x16 (&acc0)[NB], lds_cptr tile1, const i32x4 (&breg1)[HD / 16],
-                                           f32x16 (&acc1)[NB], const f32x16& init1, Hook&& hook = Hook{}) {
-  constexpr int KK = HD / 16, N = 2 * NB * KK;
-  i32x4 ops[N];
-  // step j: which = j & 1, bb = (j >> 1) % NB, kk = (j >> 1) / NB
-#pragma unroll
-  for (int j = 0; j < DEPTH && j < N; j++)
-    ops[j] = oa.row_operand((j & 1) ? tile1 : tile0, 32 * ((j >> 1) % NB), (j >> 1) / NB);
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int j = 0; j < N; j++) {
-    if (j + DEPTH < N) {
-      const int jn = j + DEPTH;
-      ops[jn] = oa.row_operand((jn & 1) ? tile1 : tile0, 32 * ((jn >> 1) % NB), (jn >> 1) / NB);
-    }
-    const int bb = (j >> 1) % NB, kk = (j >> 1) / NB;
-    f32x16 z;
-#pragma unroll
-    for (int i = 0; i < 16; i++) z[i] = 0.f;
-    if (j & 1)
-      acc1[bb] = mfma32<T>(ops[j], breg1[kk], kk == 0 ? init1 : acc1[bb]);
-    else
-      acc0[bb] = mfma32<T>(ops[j], breg0[kk], kk == 0 ? z : acc0[bb]);
-    __builtin_amdgcn_sched_barrier(0);
-    hook(j);
-  }
-}
-
 // acc[d] += tr(tile, 16*ks, d) x breg[ks]  for ks < NKS, d < HD/32.  prefetch() may be
 // called early (before the code that produces breg) to have the first operands waiting.
 template <typename T, int HD, int NKS, int DEPTH>
