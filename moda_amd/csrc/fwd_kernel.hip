@@ -35,6 +35,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   constexpr bool PP = Shape::PP;
   static_assert(NST >= DIST + 1 + (PP ? 1 : 0) && DIST >= 1 && DIST <= 2,
                 "ring must hold the tile in use, the tiles in flight and (ping-pong) the previous tile");
+  static_assert(2 * NST >= Shape::W, "the ring must be large enough for one 32-column K tile and V tile per wave");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
@@ -94,8 +95,12 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
     // last workgroup compute on zero queries there and are never stored)
     n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
   }
+  // Depth columns a wave alone can see (always outside chunk-visible mode, and in it when a chunk's rows fit a
+  // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span after the
+  // sequence tiles (see the end of the kernel).
+  const bool own_depth = a.L > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
   int dep0 = 0, n_dep = 0;
-  if (a.L > 0) {
+  if (a.L > 0 && !own_depth) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
     dep0 = lo_t * a.L;
     n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
@@ -168,15 +173,17 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   // probabilities in P; back: O^T += V^T P^T.
   i32x4 P[4];
   TrPipe<T, HD, 4, 2> pv;
-  auto front = [&](auto masked, lds_cptr Kc, int col0, int lo, int hi, auto&& after_scores) {
+  const std::integral_constant<int, 2> two{};
+  auto front = [&](auto masked, auto nblk, lds_cptr Kc, int col0, int lo, int hi, auto&& after_scores) {
     constexpr bool MASKED = decltype(masked)::value;
-    f32x16 s[2];
-    mfma_rows<T, HD, 2, 4>(oa, Kc, Qr, s);
+    constexpr int NBLK = decltype(nblk)::value;  // 32-column blocks of the tile
+    f32x16 s[NBLK];
+    mfma_rows<T, HD, NBLK, 4>(oa, Kc, Qr, s);
     after_scores();
     // row maximum of the raw scores (scale > 0, so it commutes with the max)
     float mx = kNegInf;
 #pragma unroll
-    for (int bb = 0; bb < 2; bb++)
+    for (int bb = 0; bb < NBLK; bb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         if (MASKED) {
@@ -203,7 +210,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
     const float neg_m = (m == kNegInf) ? 0.f : -m;
     float rs0 = 0.f, rs1 = 0.f;  // fp32 row sum of the unrounded probabilities, as the reference keeps it
 #pragma unroll
-    for (int bb = 0; bb < 2; bb++)
+    for (int bb = 0; bb < NBLK; bb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         float p = fast_exp2(__builtin_fmaf(s[bb][i], sc, neg_m));
@@ -218,12 +225,12 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
           rs0 += p;
       }
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
+    for (int ks = 0; ks < 2 * NBLK; ks++) P[ks] = pack8<T>(s[ks >> 1], (ks & 1) * 8);
     l += pair_sum(rs0 + rs1);
   };
   // the whole tile at once: the first V^T operands start travelling while the softmax runs
   auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, int lo, int hi) {
-    front(masked, Kc, col0, lo, hi, [&]() { pv.prefetch(oa, Vc); });
+    front(masked, two, Kc, col0, lo, hi, [&]() { pv.prefetch(oa, Vc); });
     pv.run(oa, Vc, P, o);
   };
   auto back = [&](lds_cptr Vc) {
@@ -283,7 +290,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
     // the late half: [V product of the previous tile] [scores + softmax of this tile] [barrier]
     if (n_full > 0) {  // first tile: nothing to finish yet
       if (DIST < ntiles) issue(DIST);
-      front(std::false_type{}, smem, 0, 0, 0, []() {});
+      front(std::false_type{}, two, smem, 0, 0, 0, []() {});
       wait_tile(1);
       __syncthreads();
       it = 1;
@@ -292,7 +299,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
     auto full_tile = [&](lds_cptr Vp, lds_cptr Kc) {
       if (it + DIST < ntiles) issue(it + DIST);
       back(Vp);
-      front(std::false_type{}, Kc, it * BN, 0, 0, []() {});
+      front(std::false_type{}, two, Kc, it * BN, 0, 0, []() {});
       wait_tile(it + 1);
       __syncthreads();
       it++;
@@ -324,7 +331,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
       const int hi = dep ? dhi : shi;
       const bool touches = (hi > col0) && (lo < col0 + BN) && (hi > lo);
       if (__any(touches)) {
-        front(std::true_type{}, stage_k(c_st), col0, lo, hi, []() {});
+        front(std::true_type{}, two, stage_k(c_st), col0, lo, hi, []() {});
         pending = true;
         p_st = c_st;
       }
@@ -333,6 +340,48 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
       __syncthreads();
     }
     if (pending) back(stage_k(p_st) + BN * HD);
+  }
+
+  if (own_depth) {
+    // The wave's own depth columns, 32 at a time through a wave-private K tile and V tile cut out of the ring
+    // (no workgroup barrier after the one that retires the ring).  The next K tile is fetched as soon as the
+    // scores are out, the next V tile once the V product is.
+    __syncthreads();
+    typedef WaveTileLoader<HD> Own;
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    lds_ptr Kt = smem + wv * (2 * 32 * HD), Vt = Kt + 32 * HD;
+    const int rw0 = qt * BM + wv * 32;
+    if (rw0 < a.Tq) {
+      const int tw0 = rw0 / a.Gf, tw1 = (min(a.Tq, rw0 + 32) - 1) / a.Gf;
+      const int c_beg = __builtin_amdgcn_readfirstlane((a.chunk ? (tw0 / a.Cb) * a.Cb : tw0) * a.L);
+      const int c_end = __builtin_amdgcn_readfirstlane((tw1 + 1) * a.L);
+      const int nh = (c_end - c_beg + 31) / 32;
+      const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
+      const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
+      Own own;
+      own.init(lane, a.D);
+      own.fetch(Kt, kdp, a.skd.t, c_beg, min(32, c_end - c_beg));
+      own.fetch(Vt, vdp, a.svd.t, c_beg, min(32, c_end - c_beg));
+      const std::integral_constant<int, 1> one{};
+      for (int j = 0; j < nh; j++) {
+        const int col0 = c_beg + 32 * j;
+        const bool more = j + 1 < nh;
+        Own::template wait_but<Own::N>();  // K landed, V may still be on its way
+        front(std::true_type{}, one, Kt, col0, dlo, dhi, []() {});
+        Own::reads_done();
+        if (more) own.fetch(Kt, kdp, a.skd.t, col0 + 32, min(32, c_end - col0 - 32));
+        if (more)
+          Own::template wait_but<Own::N>();  // V landed, the next K on its way
+        else
+          Own::template wait_but<0>();
+        TrPipe<T, HD, 2, 2> pv1;
+        const i32x4 P1[2] = {P[0], P[1]};
+        pv1.prefetch(oa, Vt);
+        pv1.run(oa, Vt, P1, o);
+        Own::reads_done();
+        if (more) own.fetch(Vt, vdp, a.svd.t, col0 + 32, min(32, c_end - col0 - 32));
+      }
+    }
   }
 
   if (valid) {

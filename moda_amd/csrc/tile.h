@@ -400,6 +400,46 @@ struct AsyncTileLoader {
   }
 };
 
+// A 32-row tile that ONE wave stages for itself (same swizzled layout, same zero fill past the end of the
+// source and past the tensors' head dim).  Nothing but the wave's own counters orders these loads: wait for
+// vmcnt before reading the tile, and for lgkmcnt(0) -- all LDS reads returned -- before loading over it.
+template <int HD>
+struct WaveTileLoader {
+  static constexpr int CH = HD / 8, RPW = 64 / CH, N = 32 / RPW;  // chunks per row, rows per load, loads per tile
+  int prow, pch, d;
+  __device__ __forceinline__ void init(int lane, int head_dim) {
+    prow = lane / CH;
+    pch = lane % CH;
+    d = head_dim;
+  }
+  // rows [row0, row0 + nrows) of the slice at `base` (nrows <= 32; the rest of the tile arrives as zeros)
+  __device__ __forceinline__ void fetch(lds_ptr tile, const uint16_t* base, int64_t row_stride, int64_t row0,
+                                        int nrows) const {
+    const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
+    const i32x4 rs = rsrc_words(base + row0 * row_stride, nrows > 0 ? (uint32_t)nrows * stride_bytes : 0u);
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      const int row = i * RPW + prow;
+      const int lch = pch ^ Tile<HD>::swz(row);
+      lds_dma<16>(rs, lds_addr(tile + i * 512), lch * 8 < d ? row * (int)stride_bytes + lch * 16 : 0x7ffffff0, 0);
+    }
+  }
+  // at most K of this wave's vector-memory loads (the youngest) still in flight
+  template <int K>
+  __device__ __forceinline__ static void wait_but() {
+    static_assert(K >= 0 && K < 64, "vmcnt is a 6-bit counter");
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (K & 15) | ((K >> 4) << 14));
+    asm volatile("" ::: "memory");
+  }
+  // every LDS read of this wave has returned
+  __device__ __forceinline__ static void reads_done() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    asm volatile("" ::: "memory");
+  }
+};
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Combine a value with the one held by lane ^ 32 (the other half of the lane pair that shares a
