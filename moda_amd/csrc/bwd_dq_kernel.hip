@@ -115,8 +115,12 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
     n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
   }
+  // Depth columns a wave alone can see (always outside chunk-visible mode, and in it when a chunk's rows fit a
+  // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span after the
+  // sequence tiles (see the end of the kernel).
+  const bool own_depth = a.L > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
   int dep0 = 0, n_dep = 0;
-  if (a.L > 0) {
+  if (a.L > 0 && !own_depth) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
     dep0 = lo_t * a.L;
     n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
@@ -182,14 +186,19 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   f32x4 dp_init[2];
 #pragma unroll
   for (int nb = 0; nb < 2; nb++) dp_init[nb] = f32x4{delta[nb], delta[nb], delta[nb], delta[nb]};
-  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, const int (&lo)[2], const int (&hi)[2]) {
+  // `nblk`: 16-column blocks of the tile (4, or 2 for a wave's own depth tiles); `scored` runs once K and V
+  // have been read for the scores (V is not needed after that)
+  auto tile = [&](auto masked, auto nblk, lds_cptr Kc, lds_cptr Vc, int col0, const int (&lo)[2], const int (&hi)[2],
+                  auto&& scored) {
     constexpr bool MASKED = decltype(masked)::value;
-    f32x4 s[4][2], dp[4][2];
-    mfma16_rows2<T, HD, 4, 2, 2>(oa, Kc, Qr, s, Vc, dOr, dp, dp_init);
-    TrPipe16<T, HD, 2, 2, 3> kt;
+    constexpr int MBLK = decltype(nblk)::value;
+    f32x4 s[MBLK][2], dp[MBLK][2];
+    mfma16_rows2<T, HD, MBLK, 2, 2>(oa, Kc, Qr, s, Vc, dOr, dp, dp_init);
+    scored();
+    TrPipe16<T, HD, MBLK / 2, 2, 3> kt;
     kt.prefetch(oa, Kc);
 #pragma unroll
-    for (int mb = 0; mb < 4; mb++)
+    for (int mb = 0; mb < MBLK; mb++)
 #pragma unroll
       for (int nb = 0; nb < 2; nb++)
 #pragma unroll
@@ -201,9 +210,9 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
           }
           s[mb][nb][i] = p * dp[mb][nb][i];
         }
-    i32x4 DS[2][2];
+    i32x4 DS[MBLK / 2][2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int ks = 0; ks < MBLK / 2; ks++)
 #pragma unroll
       for (int nb = 0; nb < 2; nb++) DS[ks][nb] = pack_slots<T>(s[2 * ks][nb], s[2 * ks + 1][nb]);
     kt.run(oa, Kc, DS, dq);
@@ -211,10 +220,11 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
 
   int it = 0;
   const int none[2] = {0, 0};
+  const std::integral_constant<int, 4> four{};
   for (; it < n_full; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     lds_cptr Kc = smem + c_st * 2 * BN * HD;
-    tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, none, none);
+    tile(std::false_type{}, four, Kc, Kc + BN * HD, it * BN, none, none, []() {});
     c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
     wait_tile(it + 1);
     __syncthreads();
@@ -233,11 +243,46 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     }
     if (__any(touches)) {
       lds_cptr Kc = smem + c_st * 2 * BN * HD;
-      tile(std::true_type{}, Kc, Kc + BN * HD, col0, lo, hi);
+      tile(std::true_type{}, four, Kc, Kc + BN * HD, col0, lo, hi, []() {});
     }
     c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
     wait_tile(it + 1);
     __syncthreads();
+  }
+
+  if (own_depth) {
+    // The wave's own depth columns, 32 at a time through a wave-private K tile and V tile cut out of the ring
+    // (no workgroup barrier after the one that retires the ring).  The next V tile is fetched as soon as the
+    // scores are out, the next K tile once dQ has its share.
+    __syncthreads();
+    typedef WaveTileLoader<HD> Own;
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    lds_ptr Kt = smem + wv * (2 * 32 * HD), Vt = Kt + 32 * HD;
+    const int rw0 = qt * BM + wv * 32;
+    if (rw0 < a.Tq) {
+      const int tw0 = rw0 / a.Gf, tw1 = (min(a.Tq, rw0 + 32) - 1) / a.Gf;
+      const int c_beg = __builtin_amdgcn_readfirstlane((a.chunk ? (tw0 / a.Cb) * a.Cb : tw0) * a.L);
+      const int c_end = __builtin_amdgcn_readfirstlane((tw1 + 1) * a.L);
+      const int nh = (c_end - c_beg + 31) / 32;
+      const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
+      const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
+      Own own;
+      own.init(lane, a.D);
+      own.fetch(Kt, kdp, a.skd.t, c_beg, min(32, c_end - c_beg));
+      own.fetch(Vt, vdp, a.svd.t, c_beg, min(32, c_end - c_beg));
+      const std::integral_constant<int, 2> two{};
+      for (int j = 0; j < nh; j++) {
+        const int col0 = c_beg + 32 * j;
+        const bool more = j + 1 < nh;
+        Own::template wait_but<0>();
+        tile(std::true_type{}, two, Kt, Vt, col0, dlo, dhi, [&]() {
+          Own::reads_done();
+          if (more) own.fetch(Vt, vdp, a.svd.t, col0 + 32, min(32, c_end - col0 - 32));
+        });
+        Own::reads_done();
+        if (more) own.fetch(Kt, kdp, a.skd.t, col0 + 32, min(32, c_end - col0 - 32));
+      }
+    }
   }
 
 #pragma unroll
@@ -268,7 +313,8 @@ hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
 
 template <typename T, int HD, typename Shape, int ADDR>
 hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
+  // the ring, or one 32-column K tile and V tile per wave for the waves' own depth columns
+  constexpr size_t smem = (size_t)std::max(Shape::NST * 2, Shape::W) * 64 * HD * sizeof(uint16_t);
   static LdsAttrState attr;
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dq_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;
