@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a_in) {
 }
 
 // ADDR bit 0: a (batch, head) slice is wider than 2 GiB (descriptors anchored per tile instead of 32-bit
-// offsets inside the slice); bit 1: packed variable-length batch
+// offsets inside the slice); bit 1: packed variable-length batch; bit 2: no depth stream
 template <typename T, int HD, typename Shape, int ADDR>
 __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) {
   constexpr int BM = 32 * Shape::W, BN = 64, KS = HD / 32, MB = HD / 16, NT = 64 * Shape::W, NST = Shape::NST, DIST = Shape::DIST;
@@ -61,12 +61,16 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, q4 = lane >> 4;
   constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0;
+  // bit 2: launched without a depth stream (the plain and sequence-only calls): the depth code is compiled out,
+  // so that it cannot disturb the register allocation of their main loop
+  constexpr bool NODEPTH = (ADDR & 4) != 0;
   const int BH = a_in.B * a_in.Hq;
   const int bh = blockIdx.x % BH;
   int b = bh / a_in.Hq;
   const int hq = bh % a_in.Hq, hkv = hq / a_in.hdiv;
   SeqArgs<VARLEN> seq(a_in, b);
   const KArgs& a = seq.a;
+  const int Ld = NODEPTH ? 0 : a.L;  // depth slots per token
   const int nqt = (a.Tq + BM - 1) / BM;
   const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
   if (VARLEN && qt >= nqt) return;
@@ -95,7 +99,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
       delta[nb] = a.delta[((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r];
       const int t = r / a.Gf;
       if (a.has_seq) shi[nb] = a.causal ? t + 1 : a.T;
-      if (a.L > 0) {
+      if (Ld > 0) {
         const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
         dlo[nb] = lo_t * a.L;
         dhi[nb] = a.chunk ? (t + 1) * a.L : dlo[nb] + a.Lv;
@@ -118,9 +122,9 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   // Depth columns a wave alone can see (always outside chunk-visible mode, and in it when a chunk's rows fit a
   // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span after the
   // sequence tiles (see the end of the kernel).
-  const bool own_depth = a.L > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
+  const bool own_depth = Ld > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
   int dep0 = 0, n_dep = 0;
-  if (a.L > 0 && !own_depth) {
+  if (Ld > 0 && !own_depth) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
     dep0 = lo_t * a.L;
     n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
@@ -142,13 +146,13 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   int ld_st = 0;
   auto issue = [&](int it) {
     lds_ptr Kt = smem + ld_st * 2 * BN * HD;
-    if (it == n_seq) {
+    if (!NODEPTH && it == n_seq) {
       srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
       srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
     if (WIDE) {
-      const bool dep = it >= n_seq;
+      const bool dep = !NODEPTH && it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
               row0, row_end);
@@ -231,7 +235,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   }
   for (; it < ntiles; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
-    const bool dep = it >= n_seq;
+    const bool dep = !NODEPTH && it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
     int lo[2], hi[2];
     bool touches = false;
@@ -325,6 +329,13 @@ hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <typename T, int HD, int ADDR>
+hipError_t launch_dq_t_addr(const KArgs& a, bool small, hipStream_t stream) {
+  if (ADDR & 1) return launch_dq_t_shape<T, HD, RowLarge, ADDR>(a, stream);  // slices wider than 2 GiB: never a small launch
+  if (small) return launch_dq_t_shape<T, HD, RowSmall<HD>, ADDR>(a, stream);
+  return launch_dq_t_shape<T, HD, RowLarge, ADDR>(a, stream);
+}
+
 template <typename T, int HD>
 hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
   // byte span of the widest streamed (batch, head) slice
@@ -332,40 +343,17 @@ hipError_t launch_dq_t(const KArgs& a, hipStream_t stream) {
                                     std::max((int64_t)a.T * a.L * a.skd.t, (int64_t)a.T * a.L * a.svd.t));
   const bool wide = span > 0x7fffffffll;
   const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
-  if (a.cu) {
-    if (wide) return launch_dq_t_shape<T, HD, RowLarge, 3>(a, stream);
-    if (small) return launch_dq_t_shape<T, HD, RowSmall<HD>, 2>(a, stream);
-    return launch_dq_t_shape<T, HD, RowLarge, 2>(a, stream);
+  switch ((wide ? 1 : 0) | (a.cu ? 2 : 0) | (a.L == 0 ? 4 : 0)) {
+    case 0: return launch_dq_t_addr<T, HD, 0>(a, small, stream);
+    case 1: return launch_dq_t_addr<T, HD, 1>(a, small, stream);
+    case 2: return launch_dq_t_addr<T, HD, 2>(a, small, stream);
+    case 3: return launch_dq_t_addr<T, HD, 3>(a, small, stream);
+    case 4: return launch_dq_t_addr<T, HD, 4>(a, small, stream);
+    case 5: return launch_dq_t_addr<T, HD, 5>(a, small, stream);
+    case 6: return launch_dq_t_addr<T, HD, 6>(a, small, stream);
+    default: return launch_dq_t_addr<T, HD, 7>(a, small, stream);
   }
-  if (wide) return launch_dq_t_shape<T, HD, RowLarge, 1>(a, stream);
-  if (small) return launch_dq_t_shape<T, HD, RowSmall<HD>, 0>(a, stream);
-  return launch_dq_t_shape<T, HD, RowLarge, 0>(a, stream);
 }
-
-template __global__ void dq_kernel<BF16, 128, RowLarge, 0>(const KArgs);
-template __global__ void dq_kernel<BF16, 64, RowLarge, 0>(const KArgs);
-template __global__ void dq_kernel<FP16, 128, RowLarge, 0>(const KArgs);
-template __global__ void dq_kernel<FP16, 64, RowLarge, 0>(const KArgs);
-template __global__ void dq_kernel<BF16, 128, RowLarge, 1>(const KArgs);
-template __global__ void dq_kernel<BF16, 64, RowLarge, 1>(const KArgs);
-template __global__ void dq_kernel<FP16, 128, RowLarge, 1>(const KArgs);
-template __global__ void dq_kernel<FP16, 64, RowLarge, 1>(const KArgs);
-template __global__ void dq_kernel<BF16, 128, RowSmall<128>, 0>(const KArgs);
-template __global__ void dq_kernel<BF16, 64, RowSmall<64>, 0>(const KArgs);
-template __global__ void dq_kernel<FP16, 128, RowSmall<128>, 0>(const KArgs);
-template __global__ void dq_kernel<FP16, 64, RowSmall<64>, 0>(const KArgs);
-template __global__ void dq_kernel<BF16, 128, RowLarge, 2>(const KArgs);
-template __global__ void dq_kernel<BF16, 128, RowLarge, 3>(const KArgs);
-template __global__ void dq_kernel<BF16, 128, RowSmall<128>, 2>(const KArgs);
-template __global__ void dq_kernel<BF16, 64, RowLarge, 2>(const KArgs);
-template __global__ void dq_kernel<BF16, 64, RowLarge, 3>(const KArgs);
-template __global__ void dq_kernel<BF16, 64, RowSmall<64>, 2>(const KArgs);
-template __global__ void dq_kernel<FP16, 128, RowLarge, 2>(const KArgs);
-template __global__ void dq_kernel<FP16, 128, RowLarge, 3>(const KArgs);
-template __global__ void dq_kernel<FP16, 128, RowSmall<128>, 2>(const KArgs);
-template __global__ void dq_kernel<FP16, 64, RowLarge, 2>(const KArgs);
-template __global__ void dq_kernel<FP16, 64, RowLarge, 3>(const KArgs);
-template __global__ void dq_kernel<FP16, 64, RowSmall<64>, 2>(const KArgs);
 
 hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_delta_t<BF16, 128>(a, stream);

@@ -27,7 +27,7 @@ namespace moda {
 using FwdLarge = RowLargePP;
 
 // ADDR bit 0: a (batch, head) slice is wider than 2 GiB (descriptors anchored per tile instead of 32-bit
-// offsets inside the slice); bit 1: packed variable-length batch
+// offsets inside the slice); bit 1: packed variable-length batch; bit 2: no depth stream
 template <typename T, int HD, typename Shape, int ADDR>
 __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in) {
   constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST,
@@ -41,12 +41,16 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
   constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0;
+  // bit 2: launched without a depth stream (the plain and sequence-only calls): the depth code is compiled out,
+  // so that it cannot disturb the register allocation of their main loop
+  constexpr bool NODEPTH = (ADDR & 4) != 0;
   const int BH = a_in.B * a_in.Hq;
   const int bh = blockIdx.x % BH;
   int b = bh / a_in.Hq;
   const int hq = bh % a_in.Hq, hkv = hq / a_in.hdiv;
   SeqArgs<VARLEN> seq(a_in, b);
   const KArgs& a = seq.a;
+  const int Ld = NODEPTH ? 0 : a.L;  // depth slots per token
   const int nqt = (a.Tq + BM - 1) / BM;
   // Heavy (late) tiles first.  In a variable-length batch the grid counts tiles from the end of the longest
   // sequence, so that tiles of equal cost (equal row position) of all sequences are dispatched together and the
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   int shi = 0, dlo = 0, dhi = 0;
   if (valid) {
     if (a.has_seq) shi = a.causal ? t + 1 : a.T;
-    if (a.L > 0) {
+    if (Ld > 0) {
       const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
       dlo = lo_t * a.L;
       dhi = a.chunk ? (t + 1) * a.L : dlo + a.Lv;  // the token's filled slots
@@ -98,9 +102,9 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   // Depth columns a wave alone can see (always outside chunk-visible mode, and in it when a chunk's rows fit a
   // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span after the
   // sequence tiles (see the end of the kernel).
-  const bool own_depth = a.L > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
+  const bool own_depth = Ld > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
   int dep0 = 0, n_dep = 0;
-  if (a.L > 0 && !own_depth) {
+  if (Ld > 0 && !own_depth) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
     dep0 = lo_t * a.L;
     n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
@@ -126,13 +130,13 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   int ld_st = 0;  // ring stage the next issued tile goes to
   auto issue = [&](int it) {
     lds_ptr Kt = smem + ld_st * 2 * BN * HD;
-    if (it == n_seq) {
+    if (!NODEPTH && it == n_seq) {
       srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
       srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
     if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
-      const bool dep = it >= n_seq;
+      const bool dep = !NODEPTH && it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
               row0, row_end);
@@ -273,7 +277,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
     // phase 2: boundary sequence tiles and depth tiles
     for (; it < ntiles; it++) {
       if (it + DIST < ntiles) issue(it + DIST);
-      const bool dep = it >= n_seq;
+      const bool dep = !NODEPTH && it >= n_seq;
       const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
       const int lo = dep ? dlo : 0;
       const int hi = dep ? dhi : shi;
@@ -325,7 +329,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
       if (it + DIST < ntiles) issue(it + DIST);
       if (pending) back(stage_k(p_st) + BN * HD);
       pending = false;
-      const bool dep = it >= n_seq;
+      const bool dep = !NODEPTH && it >= n_seq;
       const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
       const int lo = dep ? dlo : 0;
       const int hi = dep ? dhi : shi;
@@ -413,6 +417,13 @@ hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <typename T, int HD, int ADDR>
+hipError_t launch_fwd_t_addr(const KArgs& a, bool small, hipStream_t stream) {
+  if (ADDR & 1) return launch_fwd_t_shape<T, HD, FwdLarge, ADDR>(a, stream);  // slices wider than 2 GiB: never a small launch
+  if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, ADDR>(a, stream);
+  return launch_fwd_t_shape<T, HD, FwdLarge, ADDR>(a, stream);
+}
+
 template <typename T, int HD>
 hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
   // byte span of the widest streamed (batch, head) slice
@@ -420,40 +431,17 @@ hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
                                     std::max((int64_t)a.T * a.L * a.skd.t, (int64_t)a.T * a.L * a.svd.t));
   const bool wide = span > 0x7fffffffll;
   const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
-  if (a.cu) {
-    if (wide) return launch_fwd_t_shape<T, HD, FwdLarge, 3>(a, stream);
-    if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, 2>(a, stream);
-    return launch_fwd_t_shape<T, HD, FwdLarge, 2>(a, stream);
+  switch ((wide ? 1 : 0) | (a.cu ? 2 : 0) | (a.L == 0 ? 4 : 0)) {
+    case 0: return launch_fwd_t_addr<T, HD, 0>(a, small, stream);
+    case 1: return launch_fwd_t_addr<T, HD, 1>(a, small, stream);
+    case 2: return launch_fwd_t_addr<T, HD, 2>(a, small, stream);
+    case 3: return launch_fwd_t_addr<T, HD, 3>(a, small, stream);
+    case 4: return launch_fwd_t_addr<T, HD, 4>(a, small, stream);
+    case 5: return launch_fwd_t_addr<T, HD, 5>(a, small, stream);
+    case 6: return launch_fwd_t_addr<T, HD, 6>(a, small, stream);
+    default: return launch_fwd_t_addr<T, HD, 7>(a, small, stream);
   }
-  if (wide) return launch_fwd_t_shape<T, HD, FwdLarge, 1>(a, stream);
-  if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, 0>(a, stream);
-  return launch_fwd_t_shape<T, HD, FwdLarge, 0>(a, stream);
 }
-
-template __global__ void fwd_kernel<BF16, 128, FwdLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, FwdLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, FwdLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, FwdLarge, 0>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, FwdLarge, 1>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, FwdLarge, 1>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, FwdLarge, 1>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, FwdLarge, 1>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, 0>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, 0>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, 0>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, 0>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, FwdLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, FwdLarge, 3>(const KArgs);
-template __global__ void fwd_kernel<BF16, 128, RowSmall<128>, 2>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, FwdLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, FwdLarge, 3>(const KArgs);
-template __global__ void fwd_kernel<BF16, 64, RowSmall<64>, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, FwdLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, FwdLarge, 3>(const KArgs);
-template __global__ void fwd_kernel<FP16, 128, RowSmall<128>, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, FwdLarge, 2>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, FwdLarge, 3>(const KArgs);
-template __global__ void fwd_kernel<FP16, 64, RowSmall<64>, 2>(const KArgs);
 
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 128) return launch_fwd_t<BF16, 128>(a, stream);
