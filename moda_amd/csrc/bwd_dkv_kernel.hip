@@ -34,15 +34,20 @@ namespace moda {
 template <typename T, int HD, bool VARLEN, bool SPLIT = false>
 __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   static_assert(!(VARLEN && SPLIT), "packed batches are not split");
-  constexpr int BN = 128, BM = 64, KS = HD / 32, MB = HD / 16, NST = 3;
+  // 16-column halves per wave, query rows per streamed tile: halved for the 256-wide tiles, whose operands and
+  // accumulators would not fit the register file (and whose three-stage ring would not fit the LDS) otherwise
+  constexpr int NB = HD > 128 ? 1 : 2, BM = HD > 128 ? 32 : 64, MBLK = BM / 16;
+  constexpr int BN = 4 * 16 * NB, KS = HD / 32, MB = HD / 16, NST = 3;
+  constexpr int NP = (MBLK / 2) * NB;  // B operands of P per lane in the mailbox
+  constexpr int SP = 64;               // floats per statistic and stage (one wave-wide load each)
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
   // ring of NST stages, each: Q tile, dO tile; then the P mailbox; then lse/delta per stage
   lds_ptr ring = smem;
-  MODA_LDS i32x4* mbox = (MODA_LDS i32x4*)(smem + NST * 2 * BM * HD);      // [2 parities][4 blocks][4][64 lanes]
-  MODA_LDS float* stat = (MODA_LDS float*)(mbox + 2 * 4 * 4 * 64);         // [NST][2][BM]
+  MODA_LDS i32x4* mbox = (MODA_LDS i32x4*)(smem + NST * 2 * BM * HD);      // [2 parities][4 blocks][NP][64 lanes]
+  MODA_LDS float* stat = (MODA_LDS float*)(mbox + 2 * 4 * NP * 64);        // [NST][2][SP]
 
-  // lane (n, q4) owns columns 16*nb + n (nb = 0, 1) of the wave's block
+  // lane (n, q4) owns columns 16*nb + n (nb < NB) of the wave's block
   const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kblk = wave & 3;
@@ -71,24 +76,24 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   }
   const int c_first = tile * BN;
   if (VARLEN && c_first >= ncols) return;  // a tile beyond this sequence of a variable-length batch
-  int c[2];
-  bool valid[2], live[2];  // live: a column with data (an unwritten depth slot is seen by no row: its K/V are
+  int c[NB];
+  bool valid[NB], live[NB];  // live: a column with data (an unwritten depth slot is seen by no row: its K/V are
                            // replaced by zeros, its gradients come out zero)
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++) {
-    c[nb] = c_first + kblk * 32 + 16 * nb + n;
+  for (int nb = 0; nb < NB; nb++) {
+    c[nb] = c_first + kblk * (16 * NB) + 16 * nb + n;
     valid[nb] = c[nb] < ncols;
     live[nb] = valid[nb] && !(dep && (c[nb] % a.L) >= a.Lv);
   }
 
   // stationary operand of this wave's role: K rows (A) or V rows (B)
-  i32x4 Sr[2][KS];
+  i32x4 Sr[NB][KS];
   {
     const uint16_t* src = role_b ? (dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h)
                                  : (dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h);
     const int64_t st = role_b ? (dep ? a.svd.t : a.sv.t) : (dep ? a.skd.t : a.sk.t);
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+    for (int nb = 0; nb < NB; nb++)
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         i32x4 z = {0, 0, 0, 0};
@@ -116,10 +121,12 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
       hi = a.chunk ? min(a.T, (w / a.Cb + 1) * a.Cb) * a.Gf : (w + 1) * a.Gf;
     }
   };
-  int qlo[2] = {0, 0}, qhi[2] = {0, 0};
+  int qlo[NB], qhi[NB];
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++)
+  for (int nb = 0; nb < NB; nb++) {
+    qlo[nb] = qhi[nb] = 0;
     if (live[nb]) q_interval(c[nb], qlo[nb], qhi[nb]);
+  }
   int wg_lo, wg_hi, tmp;
   q_interval(c_first, wg_lo, tmp);
   q_interval(min(ncols, c_first + BN) - 1, tmp, wg_hi);
@@ -133,7 +140,6 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   const int niter = nqt * a.hdiv;
 
   using Loader = AsyncTileLoader<HD, BM, 512>;
-  static_assert(Loader::N == HD / 64, "one or two wave-wide loads per tile and wave");
   Loader ld;
   ld.init(tid, a.D);
   // Producer.  The global -> LDS loads of one tile are NOT issued back to back: forty wave-wide
@@ -172,7 +178,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
     rs_do = rsrc_words(do_ptr, rows * do_row_bytes);
     rs_stat = rsrc_words(st_ptr, rows > 0 ? (rows - 1) * stat_row_bytes + 4u : 0u);
     lds_q = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr(ring + ld_st * 2 * BM * HD + wave * 512));
-    lds_stat = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(stat + ld_st * 2 * BM + (wave == 0 ? 0 : BM)));
+    lds_stat = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(stat + ld_st * 2 * SP + (wave == 0 ? 0 : SP)));
     q_ptr -= (int64_t)BM * q_row_bytes;
     do_ptr -= (int64_t)BM * do_row_bytes;
     st_ptr -= (int64_t)BM * stat_row_bytes;
@@ -196,15 +202,15 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   // hook for the first MFMA phase of a tile body: one part after every third MFMA (every second one when
   // the phase is short)
   auto feed = [&](int j) {
-    constexpr int every = HD == 128 ? 3 : 2;
+    constexpr int every = HD == 64 ? 2 : 3;
     if (j % every == 1 && j / every < kParts) part(j / every);
   };
 
-  f32x4 acc[MB][2];  // dV^T (role A) or dK^T (role B): head-dim block x column block
+  f32x4 acc[MB][NB];  // dV^T (role A) or dK^T (role B): head-dim block x column block
 #pragma unroll
   for (int d = 0; d < MB; d++)
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) acc[d][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; nb++) acc[d][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float sc = a.scale * kLog2e;
   Operand16<HD> oa;
   oa.init(lane);
@@ -232,58 +238,58 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
 
   // role A, one tile: S = Q K^T, P = exp2(S c - lse) -> mailbox, dV^T += dO^T P
   auto tile_a = [&](bool masked, lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* lse_s, MODA_LDS i32x4* mb, int q0) {
-    f32x4 s[4][2];
-    mfma16_rows<T, HD, 4, 2, 4>(oa, Qs, Sr, s, feed);
-    TrPipe16<T, HD, 2, 2, 2> dvp;
+    f32x4 s[MBLK][NB];
+    mfma16_rows<T, HD, MBLK, NB, 4>(oa, Qs, Sr, s, feed);
+    TrPipe16<T, HD, MBLK / 2, NB, 2> dvp;
     dvp.prefetch(oa, dOs);
 #pragma unroll
-    for (int m = 0; m < 4; m++) {
+    for (int m = 0; m < MBLK; m++) {
       const f32x4 lv = *reinterpret_cast<MODA_LDS const f32x4*>(lse_s + 16 * m + slot_base(q4));
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++)
+      for (int nb = 0; nb < NB; nb++)
 #pragma unroll
         for (int j = 0; j < 4; j++) s[m][nb][j] = fast_exp2(__builtin_fmaf(s[m][nb][j], sc, -lv[j]));
     }
     if (masked) {  // wave-uniform; touches only s, so the accumulators stay where they are
 #pragma unroll
-      for (int m = 0; m < 4; m++)
+      for (int m = 0; m < MBLK; m++)
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++)
+        for (int nb = 0; nb < NB; nb++)
 #pragma unroll
           for (int j = 0; j < 4; j++) {
             const int qr = q0 + 16 * m + slot_base(q4) + j;
             s[m][nb][j] = (qr >= qlo[nb] && qr < qhi[nb]) ? s[m][nb][j] : 0.f;
           }
     }
-    i32x4 P[2][2];
+    i32x4 P[MBLK / 2][NB];
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int ks = 0; ks < MBLK / 2; ks++)
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++) {
+      for (int nb = 0; nb < NB; nb++) {
         P[ks][nb] = pack_slots<T>(s[2 * ks][nb], s[2 * ks + 1][nb]);
-        mb[(2 * ks + nb) * 64] = P[ks][nb];
+        mb[(NB * ks + nb) * 64] = P[ks][nb];
       }
     dvp.run(oa, dOs, P, acc);
   };
   // role B, one tile: dP - delta = dO V^T with the accumulators preset to -delta (the workspace holds
   // minus delta), dS = P (dP - delta), dK^T += Q^T dS
   auto tile_b = [&](lds_cptr Qs, lds_cptr dOs, MODA_LDS const float* del_s, MODA_LDS const i32x4* mb) {
-    f32x4 dp[4][2];
+    f32x4 dp[MBLK][NB];
 #pragma unroll
-    for (int m = 0; m < 4; m++) {
+    for (int m = 0; m < MBLK; m++) {
       const f32x4 dv = *reinterpret_cast<MODA_LDS const f32x4*>(del_s + 16 * m + slot_base(q4));
-      dp[m][0] = dv;
-      dp[m][1] = dv;
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) dp[m][nb] = dv;
     }
-    mfma16_rows<T, HD, 4, 2, 4, true>(oa, dOs, Sr, dp, feed);
-    TrPipe16<T, HD, 2, 2, 2> dkp;
+    mfma16_rows<T, HD, MBLK, NB, 4, true>(oa, dOs, Sr, dp, feed);
+    TrPipe16<T, HD, MBLK / 2, NB, 2> dkp;
     dkp.prefetch(oa, Qs);
-    i32x4 DS[2][2];
+    i32x4 DS[MBLK / 2][NB];
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int ks = 0; ks < MBLK / 2; ks++)
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++) {
-        const i32x4 pw = mb[(2 * ks + nb) * 64];
+      for (int nb = 0; nb < NB; nb++) {
+        const i32x4 pw = mb[(NB * ks + nb) * 64];
         float p[8];
 #pragma unroll
         for (int w = 0; w < 4; w++) unpack2<T>(pw[w], p[2 * w], p[2 * w + 1]);
@@ -327,12 +333,15 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
       const int st = STAGE >= 0 ? STAGE : c_st;
       lds_cptr Qs = ring + st * 2 * BM * HD;
       lds_cptr dOs = Qs + BM * HD;
-      MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * 4 * 64 + lane;
-      MODA_LDS const float* st_s = stat + st * 2 * BM;
+      MODA_LDS i32x4* mb = mbox + (c_par * 4 + kblk) * NP * 64 + lane;
+      MODA_LDS const float* st_s = stat + st * 2 * SP;
       bool run = true;
       if (MASKED) {
-        run = __any(((qhi[0] > q0) && (qlo[0] < q0 + BM) && (qhi[0] > qlo[0])) ||
-                    ((qhi[1] > q0) && (qlo[1] < q0 + BM) && (qhi[1] > qlo[1])));
+        bool touches = false;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+          touches = touches || ((qhi[nb] > q0) && (qlo[nb] < q0 + BM) && (qhi[nb] > qlo[nb]));
+        run = __any(touches);
         if (!run) {
 #pragma unroll
           for (int k = 0; k < kParts; k++) part(k);
@@ -340,7 +349,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
       }
       if (run) {
         if constexpr (ROLE_B)
-          tile_b(Qs, dOs, st_s + BM, mb);
+          tile_b(Qs, dOs, st_s + SP, mb);
         else
           tile_a(MASKED, Qs, dOs, st_s, mb, q0);
       }
@@ -383,7 +392,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
     const int64_t plane = (int64_t)a.B * a.Hkv * a.T * HD;
     const float mul = role_b ? a.scale : 1.f;
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+    for (int nb = 0; nb < NB; nb++)
       if (valid[nb]) {
         float* outp = a.dkv_part + ((int64_t)(role_b ? 0 : 1) * nseg + seg) * plane +
                       (((int64_t)b * a.Hkv + hkv) * a.T + c[nb]) * HD;
@@ -393,7 +402,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
     return;
   }
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++)
+  for (int nb = 0; nb < NB; nb++)
     if (valid[nb]) {
       uint16_t* outp;
       float mul;
@@ -729,7 +738,8 @@ __global__ __launch_bounds__(256) void dkv_reduce_kernel(const KArgs a) {
 
 template <typename T, int HD>
 hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = 3 * 2 * 64 * HD * sizeof(uint16_t) + 2 * 4 * 4 * 64 * 16 + 3 * 2 * 64 * sizeof(float);
+  constexpr int NB = HD > 128 ? 1 : 2, BM = HD > 128 ? 32 : 64, BN = 64 * NB;  // as in dkv_kernel
+  constexpr size_t smem = 3 * 2 * BM * HD * sizeof(uint16_t) + 2 * 4 * (BM / 32) * NB * 64 * 16 + 3 * 2 * 64 * sizeof(float);
   static LdsAttrState attr;
   static LdsAttrState attr_packed;
   static LdsAttrState attr_split;
@@ -741,10 +751,11 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   if (ea != hipSuccess) return ea;
   // depth columns: vector kernel, except in chunk-visible mode where a column has up to G*Cb visible rows
   const bool depth_by_columns = a.L > 0 && !a.chunk;
-  const int64_t n_seq_tiles = a.has_seq ? (a.T + 127) / 128 : 0;
-  // chunk-visible depth columns: by whole chunks when a chunk's rows fit one query tile, else as column tiles
-  const bool depth_by_chunks = a.L > 0 && a.chunk && (int64_t)a.Cb * a.Gf <= 64;
-  const int64_t n_dep_tiles = (a.L > 0 && a.chunk && !depth_by_chunks) ? ((int64_t)a.T * a.L + 127) / 128 : 0;
+  const int64_t n_seq_tiles = a.has_seq ? (a.T + BN - 1) / BN : 0;
+  // chunk-visible depth columns: by whole chunks when a chunk's rows fit one query tile (tile widths up to 128:
+  // the chunk kernel's registers and LDS do not stretch to 256), else as column tiles
+  const bool depth_by_chunks = HD <= 128 && a.L > 0 && a.chunk && (int64_t)a.Cb * a.Gf <= 64;
+  const int64_t n_dep_tiles = (a.L > 0 && a.chunk && !depth_by_chunks) ? ((int64_t)a.T * a.L + BN - 1) / BN : 0;
   const int64_t nblk = (n_seq_tiles * nseg + n_dep_tiles) * a.B * a.Hkv;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   if (nblk > 0) {
@@ -763,7 +774,7 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
       if (er != hipSuccess) return er;
     }
   }
-  if (depth_by_chunks && (int64_t)a.B * a.T > 0) {
+  if constexpr (HD <= 128) if (depth_by_chunks && (int64_t)a.B * a.T > 0) {
     constexpr size_t csmem = (2 * 64 + 4 * 32) * HD * sizeof(uint16_t) + 2 * 64 * sizeof(float);
     const int64_t nx = (((int64_t)a.T + a.Cb - 1) / a.Cb) * a.B * a.Hkv;
     if (nx >= (1ll << 31)) return hipErrorInvalidValue;
@@ -808,6 +819,8 @@ hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 64) return launch_dkv_t<BF16, 64>(a, stream);
   if (dtype == 1 && hd == 128) return launch_dkv_t<FP16, 128>(a, stream);
   if (dtype == 1 && hd == 64) return launch_dkv_t<FP16, 64>(a, stream);
+  if (dtype == 0 && hd == 256) return launch_dkv_t<BF16, 256>(a, stream);
+  if (dtype == 1 && hd == 256) return launch_dkv_t<FP16, 256>(a, stream);
   return hipErrorInvalidValue;
 }
 

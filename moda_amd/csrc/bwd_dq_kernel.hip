@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a_in) {
 // offsets inside the slice); bit 1: packed variable-length batch; bit 2: no depth stream
 template <typename T, int HD, typename Shape, int ADDR>
 __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) {
-  constexpr int BM = 32 * Shape::W, BN = 64, KS = HD / 32, MB = HD / 16, NT = 64 * Shape::W, NST = Shape::NST, DIST = Shape::DIST;
+  constexpr int NB = Shape::NB, WR = 16 * NB, BM = WR * Shape::W, BN = 64, KS = HD / 32, MB = HD / 16, NT = 64 * Shape::W, NST = Shape::NST, DIST = Shape::DIST;
   static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   lds_ptr smem = (lds_ptr)smem_raw;
@@ -75,12 +75,12 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
   if (VARLEN && qt >= nqt) return;
 
-  i32x4 Qr[2][KS], dOr[2][KS];
-  float lse[2], delta[2];
-  int shi[2], dlo[2], dhi[2];
+  i32x4 Qr[NB][KS], dOr[NB][KS];
+  float lse[NB], delta[NB];
+  int shi[NB], dlo[NB], dhi[NB];
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++) {
-    const int r = qt * BM + wave * 32 + 16 * nb + n;
+  for (int nb = 0; nb < NB; nb++) {
+    const int r = qt * BM + wave * WR + 16 * nb + n;
     const bool valid = r < a.Tq;
     const uint16_t* qp = a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + 8 * q4;
     const uint16_t* dop = a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + 8 * q4;
@@ -122,7 +122,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   // Depth columns a wave alone can see (always outside chunk-visible mode, and in it when a chunk's rows fit a
   // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span after the
   // sequence tiles (see the end of the kernel).
-  const bool own_depth = Ld > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
+  constexpr bool OWN_FITS = Shape::W * 64 * HD * 2 <= 128 * 1024;  // one 32-column K and V tile per wave
+  const bool own_depth = OWN_FITS && Ld > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
   int dep0 = 0, n_dep = 0;
   if (Ld > 0 && !own_depth) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
@@ -171,11 +172,11 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
       Loader::wait_all();
   };
 
-  f32x4 dq[MB][2];
+  f32x4 dq[MB][NB];
 #pragma unroll
   for (int d = 0; d < MB; d++)
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) dq[d][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; nb++) dq[d][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float sc = a.scale * kLog2e;
   Operand16<HD> oa;
   oa.init(lane);
@@ -187,24 +188,24 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   __syncthreads();
   int c_st = 0;
 
-  f32x4 dp_init[2];
+  f32x4 dp_init[NB];
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++) dp_init[nb] = f32x4{delta[nb], delta[nb], delta[nb], delta[nb]};
+  for (int nb = 0; nb < NB; nb++) dp_init[nb] = f32x4{delta[nb], delta[nb], delta[nb], delta[nb]};
   // `nblk`: 16-column blocks of the tile (4, or 2 for a wave's own depth tiles); `scored` runs once K and V
   // have been read for the scores (V is not needed after that)
-  auto tile = [&](auto masked, auto nblk, lds_cptr Kc, lds_cptr Vc, int col0, const int (&lo)[2], const int (&hi)[2],
+  auto tile = [&](auto masked, auto nblk, lds_cptr Kc, lds_cptr Vc, int col0, const int (&lo)[NB], const int (&hi)[NB],
                   auto&& scored) {
     constexpr bool MASKED = decltype(masked)::value;
     constexpr int MBLK = decltype(nblk)::value;
-    f32x4 s[MBLK][2], dp[MBLK][2];
-    mfma16_rows2<T, HD, MBLK, 2, 2>(oa, Kc, Qr, s, Vc, dOr, dp, dp_init);
+    f32x4 s[MBLK][NB], dp[MBLK][NB];
+    mfma16_rows2<T, HD, MBLK, NB, 2>(oa, Kc, Qr, s, Vc, dOr, dp, dp_init);
     scored();
-    TrPipe16<T, HD, MBLK / 2, 2, 3> kt;
+    TrPipe16<T, HD, MBLK / 2, NB, 3> kt;
     kt.prefetch(oa, Kc);
 #pragma unroll
     for (int mb = 0; mb < MBLK; mb++)
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++)
+      for (int nb = 0; nb < NB; nb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           float p = fast_exp2(__builtin_fmaf(s[mb][nb][i], sc, -lse[nb]));
@@ -214,16 +215,18 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
           }
           s[mb][nb][i] = p * dp[mb][nb][i];
         }
-    i32x4 DS[MBLK / 2][2];
+    i32x4 DS[MBLK / 2][NB];
 #pragma unroll
     for (int ks = 0; ks < MBLK / 2; ks++)
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++) DS[ks][nb] = pack_slots<T>(s[2 * ks][nb], s[2 * ks + 1][nb]);
+      for (int nb = 0; nb < NB; nb++) DS[ks][nb] = pack_slots<T>(s[2 * ks][nb], s[2 * ks + 1][nb]);
     kt.run(oa, Kc, DS, dq);
   };
 
   int it = 0;
-  const int none[2] = {0, 0};
+  int none[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) none[nb] = 0;
   const std::integral_constant<int, 4> four{};
   for (; it < n_full; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
@@ -237,10 +240,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     if (it + DIST < ntiles) issue(it + DIST);
     const bool dep = !NODEPTH && it >= n_seq;
     const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
-    int lo[2], hi[2];
+    int lo[NB], hi[NB];
     bool touches = false;
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
+    for (int nb = 0; nb < NB; nb++) {
       lo[nb] = dep ? dlo[nb] : 0;
       hi[nb] = dep ? dhi[nb] : shi[nb];
       touches = touches || ((hi[nb] > col0) && (lo[nb] < col0 + BN) && (hi[nb] > lo[nb]));
@@ -262,9 +265,9 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     typedef WaveTileLoader<HD> Own;
     const int wv = __builtin_amdgcn_readfirstlane(wave);
     lds_ptr Kt = smem + wv * (2 * 32 * HD), Vt = Kt + 32 * HD;
-    const int rw0 = qt * BM + wv * 32;
+    const int rw0 = qt * BM + wv * WR;
     if (rw0 < a.Tq) {
-      const int tw0 = rw0 / a.Gf, tw1 = (min(a.Tq, rw0 + 32) - 1) / a.Gf;
+      const int tw0 = rw0 / a.Gf, tw1 = (min(a.Tq, rw0 + WR) - 1) / a.Gf;
       const int c_beg = __builtin_amdgcn_readfirstlane((a.chunk ? (tw0 / a.Cb) * a.Cb : tw0) * a.L);
       const int c_end = __builtin_amdgcn_readfirstlane((tw1 + 1) * a.L);
       const int nh = (c_end - c_beg + 31) / 32;
@@ -290,8 +293,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   }
 
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++) {
-    const int r = qt * BM + wave * 32 + 16 * nb + n;
+  for (int nb = 0; nb < NB; nb++) {
+    const int r = qt * BM + wave * WR + 16 * nb + n;
     if (r < a.Tq) {
       uint16_t* op = a.dq + b * a.sdq.b + hq * a.sdq.h + (int64_t)r * a.sdq.t;
 #pragma unroll
@@ -318,11 +321,13 @@ hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
 template <typename T, int HD, typename Shape, int ADDR>
 hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
   // the ring, or one 32-column K tile and V tile per wave for the waves' own depth columns
-  constexpr size_t smem = (size_t)std::max(Shape::NST * 2, Shape::W) * 64 * HD * sizeof(uint16_t);
+  constexpr size_t ring = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t), own = (size_t)Shape::W * 64 * HD * sizeof(uint16_t);
+  constexpr size_t smem = own <= 128 * 1024 ? std::max(ring, own) : ring;
   static LdsAttrState attr;
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dq_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;
-  const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
+  constexpr int rows = 16 * Shape::NB * Shape::W;
+  const int64_t nblk = (int64_t)((a.Tq + rows - 1) / rows) * a.B * a.Hq;
   if (nblk == 0) return hipSuccess;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   hipLaunchKernelGGL((dq_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
@@ -331,9 +336,12 @@ hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
 
 template <typename T, int HD, int ADDR>
 hipError_t launch_dq_t_addr(const KArgs& a, bool small, hipStream_t stream) {
-  if (ADDR & 1) return launch_dq_t_shape<T, HD, RowLarge, ADDR>(a, stream);  // slices wider than 2 GiB: never a small launch
-  if (small) return launch_dq_t_shape<T, HD, RowSmall<HD>, ADDR>(a, stream);
-  return launch_dq_t_shape<T, HD, RowLarge, ADDR>(a, stream);
+  if constexpr (HD > 128) return launch_dq_t_shape<T, HD, RowWide, ADDR>(a, stream);  // one shape for the wide tiles
+  else {
+    if (ADDR & 1) return launch_dq_t_shape<T, HD, RowLarge, ADDR>(a, stream);  // slices wider than 2 GiB: never a small launch
+    if (small) return launch_dq_t_shape<T, HD, RowSmall<HD>, ADDR>(a, stream);
+    return launch_dq_t_shape<T, HD, RowLarge, ADDR>(a, stream);
+  }
 }
 
 template <typename T, int HD>
@@ -360,6 +368,8 @@ hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 64) return launch_delta_t<BF16, 64>(a, stream);
   if (dtype == 1 && hd == 128) return launch_delta_t<FP16, 128>(a, stream);
   if (dtype == 1 && hd == 64) return launch_delta_t<FP16, 64>(a, stream);
+  if (dtype == 0 && hd == 256) return launch_delta_t<BF16, 256>(a, stream);
+  if (dtype == 1 && hd == 256) return launch_delta_t<FP16, 256>(a, stream);
   return hipErrorInvalidValue;
 }
 
@@ -368,6 +378,8 @@ hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 64) return launch_dq_t<BF16, 64>(a, stream);
   if (dtype == 1 && hd == 128) return launch_dq_t<FP16, 128>(a, stream);
   if (dtype == 1 && hd == 64) return launch_dq_t<FP16, 64>(a, stream);
+  if (dtype == 0 && hd == 256) return launch_dq_t<BF16, 256>(a, stream);
+  if (dtype == 1 && hd == 256) return launch_dq_t<FP16, 256>(a, stream);
   return hipErrorInvalidValue;
 }
 

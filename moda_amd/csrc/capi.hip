@@ -1,5 +1,6 @@
 // C ABI of libmoda_hip.so (see include/moda_hip.h): descriptor validation and
 // dispatch to the gfx950 kernels.  No tensor-library types cross this file.
+#include <cstdlib>
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -43,13 +44,20 @@ bool row_stride_ok(const moda_hip_strides& s, int esize) { return s.t >= 0 && s.
 
 int value_dim(const moda_hip_desc* d) { return (int)(d->Dv > 0 ? d->Dv : d->D); }
 
-// The matrix-core kernels exist for tile widths 64 and 128; any 16-bit head dim that is a multiple of 8 (whole
-// 16-byte chunks) up to 128 runs on the next width, zero-padded inside the kernels.
+// The matrix-core kernels exist for tile widths 64, 128 and 256; any 16-bit head dim that is a multiple of 8 (whole
+// 16-byte chunks) up to 256 runs on the next width, zero-padded inside the kernels.
 bool use_mfma(const moda_hip_desc* d) {
-  return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && d->D % 8 == 0 && d->D <= 128 &&
+  return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && d->D % 8 == 0 && d->D <= 256 &&
          value_dim(d) == d->D;
 }
-int tile_width(const moda_hip_desc* d) { return d->D <= 64 ? 64 : 128; }
+int tile_width(const moda_hip_desc* d) { return d->D <= 64 ? 64 : d->D <= 128 ? 128 : 256; }
+// TEMPORARY while the 256-wide kernels are brought up one by one: which stages of a wide call run on them
+// (bit 0 forward, bit 1 dQ, bit 2 dK/dV), the others on the vector-ALU kernels
+bool wide_stage(const moda_hip_desc* d, int bit) {
+  if (d->D <= 128) return true;
+  const char* e = getenv("MODA_WIDE_STAGES");
+  return e && (atoi(e) & bit);
+}
 
 // Validates the descriptor and fills the geometry part of KArgs.
 int fill_geometry(const moda_hip_desc* d, KArgs& a) {
@@ -115,8 +123,9 @@ size_t delta_bytes(const KArgs& a) { return (delta_bytes_exact(a) + 255) / 256 *
 // partition mode, so that the workspace size depends on the descriptor alone.
 int desired_dkv_split(const moda_hip_desc* d, const KArgs& a) {
   if (!use_mfma(d) || a.cu || !a.has_seq || a.T == 0) return 1;
-  const int64_t tiles = (int64_t)((a.T + 127) / 128) * a.B * a.Hkv;
-  const int64_t query_tiles = (a.Tq + 63) / 64;
+  const int cols = d->D > 128 ? 64 : 128, rows = d->D > 128 ? 32 : 64;  // the kernel's column tile and query tile
+  const int64_t tiles = (int64_t)((a.T + cols - 1) / cols) * a.B * a.Hkv;
+  const int64_t query_tiles = (a.Tq + rows - 1) / rows;
   int s = 1;
   while (tiles * s < 512 && s < 8 && query_tiles / (2 * s) >= 16) s *= 2;
   return s;
@@ -217,7 +226,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
   a.skd = cvt(d->kd);
   a.svd = cvt(d->vd);
   a.so = cvt(d->o);
-  hipError_t e = use_mfma(d) ? moda::launch_fwd(a, d->dtype, tile_width(d), (hipStream_t)stream)
+  hipError_t e = use_mfma(d) && wide_stage(d, 1) ? moda::launch_fwd(a, d->dtype, tile_width(d), (hipStream_t)stream)
                              : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 0, (hipStream_t)stream);
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }
@@ -332,8 +341,12 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
   hipError_t e = hipSuccess;
   if (use_mfma(d)) {
     if (stages & MODA_HIP_STAGE_DELTA) e = moda::launch_delta(a, d->dtype, tile_width(d), s);
-    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ)) e = moda::launch_dq(a, d->dtype, tile_width(d), s);
-    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_dkv(a, d->dtype, tile_width(d), s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ))
+      e = wide_stage(d, 2) ? moda::launch_dq(a, d->dtype, tile_width(d), s)
+                           : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 1, s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV))
+      e = wide_stage(d, 4) ? moda::launch_dkv(a, d->dtype, tile_width(d), s)
+                           : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 2, s);
   } else {
     // the generic kernels recompute delta inline; the DELTA stage is a no-op for them
     if (stages & MODA_HIP_STAGE_DQ) e = moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 1, s);

@@ -3,7 +3,7 @@
 
 namespace moda {
 
-// Waves per workgroup (32 query rows each), LDS ring stages of one 64-column K tile + V tile, and how
+// Waves per workgroup (16 * NB query rows each; NB matters to the 16x16x32 kernels only), LDS ring stages of one 64-column K tile + V tile, and how
 // many tiles ahead the global->LDS loads run.
 //
 // RowLarge is the throughput shape: 256 query rows share every K/V tile.  RowSmall is for problems
@@ -13,25 +13,32 @@ namespace moda {
 // mostly the wave's own.  Its wave count is the smallest one whose tile loader covers a multiple
 // of 16 rows per pass (the LDS swizzle repeats every 16 rows).
 struct RowLarge {
-  static constexpr int W = 8, NST = 3, DIST = 2;
+  static constexpr int W = 8, NST = 3, DIST = 2, NB = 2;
   static constexpr bool PP = false;
 };
 // RowLarge with the upper half of the workgroup running half a tile behind the lower half (see the
 // forward kernel); one more ring stage keeps the previous tile's V alive for it.
 struct RowLargePP {
-  static constexpr int W = 8, NST = 4, DIST = 2;
+  static constexpr int W = 8, NST = 4, DIST = 2, NB = 2;
   static constexpr bool PP = true;
 };
 template <int HD>
 struct RowSmall;
 template <>
 struct RowSmall<64> {
-  static constexpr int W = 2, NST = 3, DIST = 2;  // 48 KB of LDS: three workgroups per compute unit
+  static constexpr int W = 2, NST = 3, DIST = 2, NB = 2;  // 48 KB of LDS: three workgroups per compute unit
   static constexpr bool PP = false;
 };
 template <>
 struct RowSmall<128> {
-  static constexpr int W = 4, NST = 2, DIST = 1;  // 64 KB of LDS: two workgroups per compute unit
+  static constexpr int W = 4, NST = 2, DIST = 1, NB = 2;  // 64 KB of LDS: two workgroups per compute unit
+  static constexpr bool PP = false;
+};
+
+// Head dims above 128 (tile width 256, 16x16x32 kernels only): 16 query rows per wave, so that the wave's Q (and
+// dO) operands and its 256-wide accumulator still fit the register file; two ring stages of 64 KB.
+struct RowWide {
+  static constexpr int W = 8, NST = 2, DIST = 1, NB = 1;
   static constexpr bool PP = false;
 };
 

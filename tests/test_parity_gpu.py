@@ -161,6 +161,14 @@ VARIANTS = [
     (1, 200, 2, 120, 3, 4, "causal", 0, torch.bfloat16),
     (2, 45, 2, 36, 3, 2, "causal", 0, torch.bfloat16),     # rows of 72 bytes: not 16-byte aligned
     (1, 40, 3, 100, 2, 1, "noncausal", 0, torch.float16),  # rows of 200 bytes
+    # head dims above 128: the 256-wide tiles (16 query rows per wave), zero-padded for 136..248
+    (1, 300, 2, 256, 5, 2, "causal", 0, torch.bfloat16),
+    (1, 260, 2, 256, 0, 4, "causal", 0, torch.bfloat16),
+    (2, 130, 2, 192, 6, 4, "chunk_visible", 16, torch.float16),
+    (1, 700, 1, 256, 3, 2, "chunk_visible", 64, torch.bfloat16),
+    (1, 197, 3, 160, 12, 1, "noncausal", 0, torch.bfloat16),
+    (1, 100, 2, 256, 7, 4, "depth_only", 0, torch.float16),
+    (1, 150, 1, 136, 2, 2, "causal", 0, torch.float16),
 ]
 
 
