@@ -36,6 +36,9 @@ WORKLOADS = {
     "plain": (1, 65536, 4, 4, 128, 0, "plain", 0),
     # c2 with a head dim between the matrix kernels' tile widths (runs zero-padded to 128)
     "c2d96": (2, 4096, 4, 4, 96, 8, "causal", 0),
+    # c2 with head dims above 128 (the 256-wide tiles; 192 runs zero-padded)
+    "c2d256": (2, 4096, 4, 4, 256, 8, "causal", 0),
+    "c2d192": (2, 4096, 4, 4, 192, 8, "causal", 0),
     # the last block of the reference's smallest MoDA vision model (4 query heads on 1 kv head, 11 earlier layers)
     "deit_tiny": (64, 197, 1, 4, 64, 11, "noncausal", 0),
     "plain_c2": (2, 4096, 4, 4, 128, 0, "plain", 0),

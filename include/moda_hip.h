@@ -5,7 +5,7 @@
  *
  * Every pointer that names tensor data is a DEVICE pointer.  Strides are in
  * elements; the innermost (head-dim) stride is always 1.  For the matrix-core
- * kernels (bf16/fp16, head dim 64 or 128, Dv == D) every row must be 16-byte
+ * kernels (bf16/fp16, head dim a multiple of 8 up to 256, Dv == D) every row must be 16-byte
  * aligned (base pointer and all strides multiples of 8 elements) and a row
  * stride must stay below 16 MiB; every other combination runs on vector-ALU
  * kernels that need element alignment only.  All work is enqueued on the hipStream_t passed

@@ -1,6 +1,5 @@
 // C ABI of libmoda_hip.so (see include/moda_hip.h): descriptor validation and
 // dispatch to the gfx950 kernels.  No tensor-library types cross this file.
-#include <cstdlib>
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -51,13 +50,6 @@ bool use_mfma(const moda_hip_desc* d) {
          value_dim(d) == d->D;
 }
 int tile_width(const moda_hip_desc* d) { return d->D <= 64 ? 64 : d->D <= 128 ? 128 : 256; }
-// TEMPORARY while the 256-wide kernels are brought up one by one: which stages of a wide call run on them
-// (bit 0 forward, bit 1 dQ, bit 2 dK/dV), the others on the vector-ALU kernels
-bool wide_stage(const moda_hip_desc* d, int bit) {
-  if (d->D <= 128) return true;
-  const char* e = getenv("MODA_WIDE_STAGES");
-  return e && (atoi(e) & bit);
-}
 
 // Validates the descriptor and fills the geometry part of KArgs.
 int fill_geometry(const moda_hip_desc* d, KArgs& a) {
@@ -226,7 +218,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
   a.skd = cvt(d->kd);
   a.svd = cvt(d->vd);
   a.so = cvt(d->o);
-  hipError_t e = use_mfma(d) && wide_stage(d, 1) ? moda::launch_fwd(a, d->dtype, tile_width(d), (hipStream_t)stream)
+  hipError_t e = use_mfma(d) ? moda::launch_fwd(a, d->dtype, tile_width(d), (hipStream_t)stream)
                              : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 0, (hipStream_t)stream);
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }
@@ -341,12 +333,8 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
   hipError_t e = hipSuccess;
   if (use_mfma(d)) {
     if (stages & MODA_HIP_STAGE_DELTA) e = moda::launch_delta(a, d->dtype, tile_width(d), s);
-    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ))
-      e = wide_stage(d, 2) ? moda::launch_dq(a, d->dtype, tile_width(d), s)
-                           : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 1, s);
-    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV))
-      e = wide_stage(d, 4) ? moda::launch_dkv(a, d->dtype, tile_width(d), s)
-                           : moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 2, s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ)) e = moda::launch_dq(a, d->dtype, tile_width(d), s);
+    if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_dkv(a, d->dtype, tile_width(d), s);
   } else {
     // the generic kernels recompute delta inline; the DELTA stage is a no-op for them
     if (stages & MODA_HIP_STAGE_DQ) e = moda::launch_generic(a, d->dtype, (int)d->D, value_dim(d), 1, s);

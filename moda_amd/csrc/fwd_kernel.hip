@@ -19,6 +19,7 @@
 
 #include "kargs.h"
 #include "tile.h"
+#include "tile16.h"
 #include "tuning.h"
 
 namespace moda {
@@ -404,6 +405,286 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   }
 }
 
+// The forward kernel for the 256-wide tiles (head dims above 128), on the 16x16x32 matrix instruction: a wave
+// owns 16 * NB query rows (NB = 1 here: Q and the 256-wide O accumulator of 32 rows would not fit the register
+// file), lane (n, q) owns rows 16*nb + n and, inside a 16-column score block, columns slot_base(q) .. +3; four
+// lanes share a row, their shares of the row sum are added at the end.  Same streaming structure and the same
+// arithmetic as fwd_kernel (which stays on 32x32x16: on the narrower tiles it is the faster of the two); depth
+// columns always stream through the workgroup's ring.
+template <typename T, int HD, typename Shape, int ADDR>
+__global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs a_in) {
+  constexpr int NB = Shape::NB, WR = 16 * NB, BM = WR * Shape::W, BN = 64, KS = HD / 32, MB = HD / 16, NT = 64 * Shape::W, NST = Shape::NST,
+                DIST = Shape::DIST;
+  static_assert(!Shape::PP, "no ping-pong schedule here");
+  static_assert(NST >= DIST + 1 && DIST >= 1 && DIST <= 2, "ring must hold the tile in use plus the tiles in flight");
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  lds_ptr smem = (lds_ptr)smem_raw;  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, q4 = lane >> 4;
+  constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0;
+  const int BH = a_in.B * a_in.Hq;
+  const int bh = blockIdx.x % BH;
+  int b = bh / a_in.Hq;
+  const int hq = bh % a_in.Hq, hkv = hq / a_in.hdiv;
+  SeqArgs<VARLEN> seq(a_in, b);
+  const KArgs& a = seq.a;
+  const int nqt = (a.Tq + BM - 1) / BM;
+  // Heavy (late) tiles first.  In a variable-length batch the grid counts tiles from the end of the longest
+  // sequence, so that tiles of equal cost (equal row position) of all sequences are dispatched together and the
+  // heaviest of the whole batch first; the positions a shorter sequence does not have are dropped.
+  const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
+  if (VARLEN && qt >= nqt) return;
+  i32x4 Qr[NB][KS];
+  int shi[NB], dlo[NB], dhi[NB];  // per-row visible column intervals [lo, hi) for the two phases
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    const int r = qt * BM + wave * WR + 16 * nb + n;
+    const bool valid = r < a.Tq;
+    const uint16_t* qp = a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + 8 * q4;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      i32x4 z = {0, 0, 0, 0};
+      Qr[nb][ks] = (valid && 32 * ks + 8 * q4 < a.D) ? *reinterpret_cast<const i32x4*>(qp + 32 * ks) : z;
+    }
+    shi[nb] = dlo[nb] = dhi[nb] = 0;
+    if (valid) {
+      const int t = r / a.Gf;
+      if (a.has_seq) shi[nb] = a.causal ? t + 1 : a.T;
+      if (a.L > 0) {
+        const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
+        dlo[nb] = lo_t * a.L;
+        dhi[nb] = a.chunk ? (t + 1) * a.L : dlo[nb] + a.Lv;  // the token's filled slots
+      }
+    }
+  }
+
+  // The register operands above must have arrived before the tile loads start: those are issued
+  // behind the compiler's back, and a load it still believes pending would cost a vmcnt(0) in every
+  // trip of the main loop.
+  asm volatile("" ::: "memory");  // keep the loads above this point
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("" ::: "memory");
+
+  // workgroup column ranges
+  const int r_first = qt * BM;
+  const int r_last = min(a.Tq, r_first + BM) - 1;
+  const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
+  int n_seq = 0, n_full = 0;
+  if (a.has_seq) {
+    n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
+    // leading sequence tiles that every row of the workgroup sees completely (padding rows of the
+    // last workgroup compute on zero queries there and are never stored)
+    n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
+  }
+  int dep0 = 0, n_dep = 0;
+  if (a.L > 0) {
+    const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
+    dep0 = lo_t * a.L;
+    n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
+  }
+  // wave-uniform by construction, but computed with vector divisions: the explicit hint keeps the
+  // loop control in scalar registers
+  n_seq = __builtin_amdgcn_readfirstlane(n_seq);
+  n_full = __builtin_amdgcn_readfirstlane(n_full);
+  dep0 = __builtin_amdgcn_readfirstlane(dep0);
+  const int ntiles = __builtin_amdgcn_readfirstlane(n_seq + n_dep);
+
+  typedef AsyncTileLoader<HD, BN, NT> Loader;
+  constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
+  Loader ld;
+  ld.init(tid, a.D);
+  // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
+  // producer reaches the first depth tile
+  typename Loader::Source srcK, srcV;
+  if (a.has_seq && n_seq > 0) {
+    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
+    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
+  }
+  int ld_st = 0;  // ring stage the next issued tile goes to
+  auto issue = [&](int it) {
+    lds_ptr Kt = smem + ld_st * 2 * BN * HD;
+    if (it == n_seq) {
+      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
+      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
+    }
+    const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
+    if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
+      const bool dep = it >= n_seq;
+      const int row_end = dep ? a.T * a.L : a.T;
+      ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
+              row0, row_end);
+      ld.load(Kt + BN * HD, dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h,
+              dep ? a.svd.t : a.sv.t, row0, row_end);
+    } else {
+      ld.load_from(Kt, srcK, row0);
+      ld.load_from(Kt + BN * HD, srcV, row0);
+    }
+    ld_st = (ld_st + 1 == NST) ? 0 : ld_st + 1;
+  };
+  // wait until tile `next` has landed; tiles next+1 .. next+DIST-1 may still be in flight
+  auto wait_tile = [&](int next) {
+    if (DIST == 2 && next + 1 < ntiles)
+      Loader::template wait_but<LPT>();
+    else
+      Loader::wait_all();
+  };
+
+  f32x4 o[MB][NB];
+#pragma unroll
+  for (int d = 0; d < MB; d++)
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) o[d][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // exponent reference (shared by the four lanes of a row) and this lane's share of the row sum
+  float m[NB], l[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    m[nb] = kNegInf;
+    l[nb] = 0.f;
+  }
+  const float sc = a.scale * kLog2e;
+  Operand16<HD> oa;
+  oa.init(lane);
+
+#pragma unroll
+  for (int j = 0; j < DIST; j++)
+    if (j < ntiles) issue(j);
+  wait_tile(0);
+  __syncthreads();
+  int c_st = 0;  // ring stage of the tile being consumed
+
+  // One column tile in two halves.  front: S^T = K Q^T and the online softmax, leaving the rounded
+  // probabilities in P; back: O^T += V^T P^T.
+  i32x4 P[2][NB];
+  TrPipe16<T, HD, 2, NB, 2> pv;
+  auto front = [&](auto masked, lds_cptr Kc, int col0, const int (&lo)[NB], const int (&hi)[NB], auto&& after_scores) {
+    constexpr bool MASKED = decltype(masked)::value;
+    f32x4 s[4][NB];
+    mfma16_rows<T, HD, 4, NB, 4>(oa, Kc, Qr, s);
+    after_scores();
+    // this lane's maximum of the raw scores of each row (scale > 0, so it commutes with the max)
+    float mx[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) mx[nb] = kNegInf;
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          if (MASKED) {
+            const int c = col0 + 16 * mb + slot_base(q4) + i;
+            mx[nb] = fmaxf(mx[nb], (c >= lo[nb] && c < hi[nb]) ? s[mb][nb][i] : kNegInf);
+          } else {
+            mx[nb] = fmaxf(mx[nb], s[mb][nb][i]);
+          }
+        }
+    bool grows = false;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      mx[nb] *= sc;
+      grows = grows || mx[nb] > m[nb] + 8.f;
+    }
+    // The exponent reference m only moves when some score outgrows it by more than 2^8:
+    // p stays <= 256, exact in fp32 accumulation and harmless in the 16-bit P, and the row-wide
+    // maximum and the rescale of O are skipped on almost every tile.
+    if (__any(grows)) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        const float m_new = fmaxf(m[nb], quad_max(mx[nb]));
+        const float alpha = fast_exp2(m[nb] - ((m_new == kNegInf) ? 0.f : m_new));
+        l[nb] *= alpha;
+        m[nb] = m_new;
+#pragma unroll
+        for (int d = 0; d < MB; d++) o[d][nb] *= alpha;
+      }
+    }
+    float rs[NB][2];  // fp32 row sum of the unrounded probabilities, as the reference keeps it
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) rs[nb][0] = rs[nb][1] = 0.f;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      const float neg_m = (m[nb] == kNegInf) ? 0.f : -m[nb];
+#pragma unroll
+      for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float p = fast_exp2(__builtin_fmaf(s[mb][nb][i], sc, neg_m));
+          if (MASKED) {
+            const int c = col0 + 16 * mb + slot_base(q4) + i;
+            p = (c >= lo[nb] && c < hi[nb]) ? p : 0.f;
+          }
+          s[mb][nb][i] = p;
+          rs[nb][i & 1] += p;
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) P[ks][nb] = pack_slots<T>(s[2 * ks][nb], s[2 * ks + 1][nb]);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) l[nb] += rs[nb][0] + rs[nb][1];
+  };
+  // the whole tile at once: the first V^T operands start travelling while the softmax runs
+  auto tile = [&](auto masked, lds_cptr Kc, lds_cptr Vc, int col0, const int (&lo)[NB], const int (&hi)[NB]) {
+    front(masked, Kc, col0, lo, hi, [&]() { pv.prefetch(oa, Vc); });
+    pv.run(oa, Vc, P, o);
+  };
+  auto stage_k = [&](int st) { return smem + st * 2 * BN * HD; };
+
+  int none[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) none[nb] = 0;
+  // phase 1: tiles fully visible to every row -- no masks, no visibility tests
+  int it = 0;
+  for (; it < n_full; it++) {
+    if (it + DIST < ntiles) issue(it + DIST);
+    lds_cptr Kc = stage_k(c_st);
+    tile(std::false_type{}, Kc, Kc + BN * HD, it * BN, none, none);
+    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    wait_tile(it + 1);
+    __syncthreads();
+  }
+  // phase 2: boundary sequence tiles and depth tiles
+  for (; it < ntiles; it++) {
+    if (it + DIST < ntiles) issue(it + DIST);
+    const bool dep = it >= n_seq;
+    const int col0 = dep ? dep0 + (it - n_seq) * BN : it * BN;
+    int lo[NB], hi[NB];
+    bool touches = false;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      lo[nb] = dep ? dlo[nb] : 0;
+      hi[nb] = dep ? dhi[nb] : shi[nb];
+      touches = touches || ((hi[nb] > col0) && (lo[nb] < col0 + BN) && (hi[nb] > lo[nb]));
+    }
+    if (__any(touches)) {
+      lds_cptr Kc = stage_k(c_st);
+      tile(std::true_type{}, Kc, Kc + BN * HD, col0, lo, hi);
+    }
+    c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
+    wait_tile(it + 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    const int r = qt * BM + wave * WR + 16 * nb + n;
+    const float lsum = quad_sum(l[nb]);
+    if (r < a.Tq) {
+      const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+      uint16_t* op = a.out_o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t;
+#pragma unroll
+      for (int d = 0; d < MB; d++) {
+        i32x2 w;
+        w[0] = pack2<T>(o[d][nb][0] * inv, o[d][nb][1] * inv);
+        w[1] = pack2<T>(o[d][nb][2] * inv, o[d][nb][3] * inv);
+        if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(op + 16 * d + 4 * q4) = w;
+      }
+      if (q4 == 0) a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq] = (lsum > 0.f) ? m[nb] + log2f(lsum) : kNegInf;
+    }
+  }
+}
+
 template <typename T, int HD, typename Shape, int ADDR>
 hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
@@ -418,10 +699,29 @@ hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
 }
 
 template <typename T, int HD, int ADDR>
+hipError_t launch_fwd_wide(const KArgs& a, hipStream_t stream) {
+  typedef RowWide Shape;
+  constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
+  static LdsAttrState attr;
+  const hipError_t ea =
+      allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_wide_kernel<T, HD, Shape, ADDR>), smem);
+  if (ea != hipSuccess) return ea;
+  constexpr int rows = 16 * Shape::NB * Shape::W;
+  const int64_t nblk = (int64_t)((a.Tq + rows - 1) / rows) * a.B * a.Hq;
+  if (nblk == 0) return hipSuccess;
+  if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((fwd_wide_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
+  return hipGetLastError();
+}
+
+template <typename T, int HD, int ADDR>
 hipError_t launch_fwd_t_addr(const KArgs& a, bool small, hipStream_t stream) {
-  if (ADDR & 1) return launch_fwd_t_shape<T, HD, FwdLarge, ADDR>(a, stream);  // slices wider than 2 GiB: never a small launch
-  if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, ADDR>(a, stream);
-  return launch_fwd_t_shape<T, HD, FwdLarge, ADDR>(a, stream);
+  if constexpr (HD > 128) return launch_fwd_wide<T, HD, ADDR & 3>(a, stream);
+  else {
+    if (ADDR & 1) return launch_fwd_t_shape<T, HD, FwdLarge, ADDR>(a, stream);  // slices wider than 2 GiB: never a small launch
+    if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, ADDR>(a, stream);
+    return launch_fwd_t_shape<T, HD, FwdLarge, ADDR>(a, stream);
+  }
 }
 
 template <typename T, int HD>
@@ -448,6 +748,8 @@ hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream) {
   if (dtype == 0 && hd == 64) return launch_fwd_t<BF16, 64>(a, stream);
   if (dtype == 1 && hd == 128) return launch_fwd_t<FP16, 128>(a, stream);
   if (dtype == 1 && hd == 64) return launch_fwd_t<FP16, 64>(a, stream);
+  if (dtype == 0 && hd == 256) return launch_fwd_t<BF16, 256>(a, stream);
+  if (dtype == 1 && hd == 256) return launch_fwd_t<FP16, 256>(a, stream);
   return hipErrorInvalidValue;
 }
 

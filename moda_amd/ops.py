@@ -94,7 +94,7 @@ def _usable(x: Optional[torch.Tensor], vec16: bool = True) -> Optional[torch.Ten
 
 
 def _matrix_core_path(q: torch.Tensor, val: torch.Tensor) -> bool:
-    """Whether the call runs on the matrix-core kernels (16-bit, head dim a multiple of 8 up to 128, the same for
+    """Whether the call runs on the matrix-core kernels (16-bit, head dim a multiple of 8 up to 256, the same for
     keys and values)."""
     return (q.dtype in (torch.bfloat16, torch.float16) and q.shape[3] % 8 == 0 and q.shape[3] <= 256
             and val.shape[3] == q.shape[3])

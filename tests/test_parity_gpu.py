@@ -1148,14 +1148,14 @@ def test_random_sweep(gpu_device, seed):
     compare_all(got, ref, dtype, f"sweep {seed}")
 
 
-def _random_case_wide(seed):
+def _random_case_wide(seed, dims=(8, 32, 64, 72, 96, 128)):
     """A second family: head dims below the tile widths, sequences long enough for the row split of the dK/dV
     kernel, chunks above and below one query tile."""
     import random
 
     rnd = random.Random(seed)
     mode = rnd.choice(["causal", "noncausal", "chunk_visible", "chunk_visible", "depth_only"])
-    D = rnd.choice([8, 32, 64, 72, 96, 128])
+    D = rnd.choice(list(dims))
     G = rnd.choice([1, 2, 4, 8, 16])
     H = rnd.choice([1, 2])
     L = rnd.choice([0, 1, 3, 6]) if mode != "depth_only" else rnd.choice([1, 3, 6])
@@ -1172,11 +1172,14 @@ def _random_case_wide(seed):
     return mode, D, G, H, L, dtype, T, B, cb, valid
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(64))
 def test_random_sweep_wide(gpu_device, seed):
+    """Seeds 40 and up draw head dims above 128 (the 256-wide tiles: 16 query rows per wave, 64-column workgroups
+    and 32-row query tiles in the dK/dV kernel)."""
     from moda_amd import ops
 
-    mode, D, G, H, L, dtype, T, B, cb, valid = _random_case_wide(5000 + seed)
+    dims = (8, 32, 64, 72, 96, 128) if seed < 40 else (136, 160, 192, 200, 256, 256)
+    mode, D, G, H, L, dtype, T, B, cb, valid = _random_case_wide(5000 + seed, dims)
     say(f"[wide sweep {seed}] mode={mode} D={D} G={G} H={H} L={L} {dtype} T={T} B={B} cb={cb} valid={valid}")
     inp = oracle.make_inputs(B, T, H, D, L, G, seed=seed, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
     sc = D ** -0.5
