@@ -264,7 +264,7 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # what FETCH_SIZE / WRITE_SIZE (KiB per dispatch) read for a plain copy of known size (the depth reorganisation
 # kernel of the same runs): FETCH_SIZE counts half of the bytes read, WRITE_SIZE all bytes written
 PMC_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
-KERNEL_NAMES = ("fwd_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "dkv_reduce_kernel", "depth_cols_kernel",
+KERNEL_NAMES = ("fwd_kernel", "fwd_wide_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "dkv_reduce_kernel", "depth_cols_kernel",
                 "chunk_depth_kernel", "reorg_kernel")
 
 

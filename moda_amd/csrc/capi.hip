@@ -45,9 +45,12 @@ int value_dim(const moda_hip_desc* d) { return (int)(d->Dv > 0 ? d->Dv : d->D); 
 
 // The matrix-core kernels exist for tile widths 64, 128 and 256; any 16-bit head dim that is a multiple of 8 (whole
 // 16-byte chunks) up to 256 runs on the next width, zero-padded inside the kernels.
+// Packed variable-length batches with head dims above 128 stay on the vector-ALU kernels: the combination of the
+// 256-wide tiles, a packed batch and chunk-visible mode ended in a GPU memory fault whose cause has not been
+// found, so the whole packed + wide path is switched off until it is.
 bool use_mfma(const moda_hip_desc* d) {
   return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && d->D % 8 == 0 && d->D <= 256 &&
-         value_dim(d) == d->D;
+         value_dim(d) == d->D && !(d->D > 128 && d->cu_seqlens);
 }
 int tile_width(const moda_hip_desc* d) { return d->D <= 64 ? 64 : d->D <= 128 ? 128 : 256; }
 

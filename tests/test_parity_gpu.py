@@ -868,6 +868,10 @@ PACKED = [
     ((3, 2, 1, 1, 40), 2, 64, 0, 2, "causal", 0, torch.bfloat16),
     ((70, 9, 31), 2, 32, 3, 2, "causal", 0, torch.float32),
     ((40, 55), 1, 96, 2, 1, "noncausal", 0, torch.bfloat16),
+    # the 256-wide tiles
+    ((130, 1, 0, 300, 65), 2, 256, 3, 2, "causal", 0, torch.bfloat16),
+    ((70, 200, 33), 1, 192, 5, 4, "chunk_visible", 8, torch.float16),
+    ((100, 7, 260), 2, 160, 4, 1, "depth_only", 0, torch.bfloat16),
 ]
 
 
