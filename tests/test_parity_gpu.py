@@ -868,6 +868,10 @@ PACKED = [
     ((3, 2, 1, 1, 40), 2, 64, 0, 2, "causal", 0, torch.bfloat16),
     ((70, 9, 31), 2, 32, 3, 2, "causal", 0, torch.float32),
     ((40, 55), 1, 96, 2, 1, "noncausal", 0, torch.bfloat16),
+    # chunks below and above one query tile (the waves' own depth phase and the chunk kernel; depth tiles streamed
+    # by the workgroup and depth column tiles in the dK/dV kernel)
+    ((70, 200, 33), 1, 128, 5, 4, "chunk_visible", 8, torch.float16),
+    ((130, 17, 400), 2, 64, 3, 4, "chunk_visible", 32, torch.bfloat16),
     # the 256-wide tiles
     ((130, 1, 0, 300, 65), 2, 256, 3, 2, "causal", 0, torch.bfloat16),
     ((70, 200, 33), 1, 192, 5, 4, "chunk_visible", 8, torch.float16),
