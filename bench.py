@@ -37,6 +37,8 @@ WORKLOADS = {
     # c2 with a head dim between the matrix kernels' tile widths (runs zero-padded to 128)
     "c2d96": (2, 4096, 4, 4, 96, 8, "causal", 0),
     # c2 with head dims above 128 (the 256-wide tiles; 192 runs zero-padded)
+    # the c3 token count with head dim 64 (the 64-wide tiles on a compute-bound shape)
+    "c3d64": (1, 16384, 4, 4, 64, 24, "causal", 0),
     "c2d256": (2, 4096, 4, 4, 256, 8, "causal", 0),
     "c2d192": (2, 4096, 4, 4, 192, 8, "causal", 0),
     # the last block of the reference's smallest MoDA vision model (4 query heads on 1 kv head, 11 earlier layers)

@@ -115,7 +115,14 @@ __device__ __forceinline__ float to_float(typename T::elem x) {
 template <int HD>
 struct Tile {
   static constexpr int CH = HD / 8;  // 16-byte chunks per row
-  __device__ __forceinline__ static int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (CH - 1); }
+  // Rows of 256 bytes and more start at bank 0 each, so all four low row bits go into the chunk index.  A 128-byte
+  // row (HD = 64) covers half the banks and odd rows the other half: there row bits 1..3 choose among the eight
+  // chunks, bit 1 on top so that rows r and r + 2 of a four-row, four-chunk transposed read land in different
+  // halves of the row.  (Measured with SQ_LDS_BANK_CONFLICT on all four operand read patterns: 0 for HD = 64,
+  // 128 and 256; the first formula cut to three bits cost HD = 64 a second pass on every read.)
+  __device__ __forceinline__ static int swz(int row) {
+    return CH == 8 ? ((((row >> 1) & 1) << 2) | ((row >> 2) & 3)) : ((((row & 3) << 2) | ((row >> 2) & 3)) & (CH - 1));
+  }
   // element offset of logical (row, chunk)
   __device__ __forceinline__ static int off(int row, int chunk) { return row * HD + ((chunk ^ swz(row)) << 3); }
 };

@@ -1,6 +1,7 @@
 // MFMA 16x16x32 building blocks.  On gfx950 the matrix pipe is power limited, and on random operands
 // the 16x16x32 shape sustains about 16 % more FLOP/s than 32x32x16 at the same operand traffic (it moves
-// a quarter of the accumulator bits per multiply-add), so the attention kernels are built on it.
+// a quarter of the accumulator bits per multiply-add), so the backward kernels and the 256-wide forward kernel
+// are built on it (the narrower forward kernel is bound by its vector work and stays on 32x32x16).
 //
 // Register layouts, lane l = (n, q) with n = l & 15, q = l >> 4:
 //   A (16 x 32):  row n,    k slots 8q .. 8q+7
