@@ -609,6 +609,27 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
 // head dim each), a wave covers 8 (D = 64) or 4 (D = 128) consecutive columns, everything stays in
 // registers and the kernel streams kd, vd in and dkd, dvd out once: it is bound by HBM.
 // P and dS are rounded to the input type before they are used, as in the matrix kernels.
+// Sum over the LPC (8, 16 or 32) consecutive lanes that share a column, result in every one of them.  The first
+// four steps are data-parallel-primitive moves inside the vector ALU (two quad permutes leave every lane of a quad
+// with the quad's sum, mirroring half a row, then the row, brings in the other quads' sums); only the step across
+// two rows of 16 lanes goes through the LDS crossbar.
+template <int LPC>
+__device__ __forceinline__ float group_sum(float x) {
+  static_assert(LPC == 8 || LPC == 16 || LPC == 32, "8, 16 or 32 lanes per column");
+#if defined(__HIP_DEVICE_COMPILE__)
+  auto dpp = [](float v, auto ctrl) {
+    const int i = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, decltype(ctrl)::value, 0xf, 0xf, false));
+  };
+  x += dpp(x, std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+  x += dpp(x, std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+  x += dpp(x, std::integral_constant<int, 0x141>{});  // row_half_mirror
+  if (LPC >= 16) x += dpp(x, std::integral_constant<int, 0x140>{});  // row_mirror
+  if (LPC == 32) x += __shfl_xor(x, 16, 64);
+#endif
+  return x;
+}
+
 template <typename T, int HD>
 __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   constexpr int LPC = HD / 8, CPW = 64 / LPC, CPB = 4 * CPW;
@@ -658,11 +679,8 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
       s = __builtin_fmaf(qf[i], kf[i], s);
       dp = __builtin_fmaf(dof[i], vf[i], dp);
     }
-#pragma unroll
-    for (int m = 1; m < LPC; m <<= 1) {
-      s += __shfl_xor(s, m, 64);
-      dp += __shfl_xor(dp, m, 64);
-    }
+    s = group_sum<LPC>(s);
+    dp = group_sum<LPC>(dp);
     const float lse = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hkv];
     const float neg_delta = a.delta[((int64_t)b * a.Hq + hkv) * a.delta_pitch + r];
     float p = fast_exp2(__builtin_fmaf(s, sc, -lse));
