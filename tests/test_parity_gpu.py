@@ -908,6 +908,32 @@ def test_packed_variable_length_batches(gpu_device, case):
     compare_all(got, ref, dtype, str(case))
 
 
+def _random_packed_case(seed):
+    import random
+
+    rnd = random.Random(seed)
+    mode = rnd.choice(["causal", "noncausal", "chunk_visible", "chunk_visible", "depth_only"])
+    D = rnd.choice([32, 64, 64, 96, 128, 128])
+    G = rnd.choice([1, 2, 4, 8])
+    H = rnd.choice([1, 2])
+    L = rnd.choice([0, 2, 5]) if mode != "depth_only" else rnd.choice([2, 5])
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    n = rnd.randint(1, 5)
+    cap = 1600 // G  # keeps every sequence's dense oracle small
+    lengths = tuple(rnd.choice([0, 1, 17, 64, 65, 130, 200, 333, 400][: 9 if cap >= 400 else 7]) for _ in range(n))
+    if sum(lengths) == 0:
+        lengths = lengths + (33,)
+    cb = rnd.choice([1, 8, 16, max(1, 64 // G), max(1, 128 // G), 40]) if mode == "chunk_visible" else 0
+    return lengths, H, D, L, G, mode, cb, dtype
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_sweep_packed(gpu_device, seed):
+    """Random packed batches on the 64- and 128-wide tiles: empty and one-token sequences, chunks below and above
+    one query tile, every mode."""
+    test_packed_variable_length_batches(gpu_device, _random_packed_case(7000 + seed))
+
+
 def test_packed_batch_equals_separate_calls_bitwise(gpu_device):
     """One launch over the packed batch returns, bit for bit, what one call per sequence returns; also
     through the public autograd interface with an int64 cu_seqlens as callers of fla pass it."""
