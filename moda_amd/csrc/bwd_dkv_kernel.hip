@@ -488,7 +488,7 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
     for (int i = 0; i < NPASS; i++) {
       const int row = i * RPW + prow;
       const int lch = pch ^ Tile<HD>::swz(row);  // chunks beyond the head dim: out of range, filled with zeros
-      lds_dma<16>(rs, lds_addr(wt + i * 512), lch * 8 < a.D ? row * (int)stride * 2 + lch * 16 : Loader::kPadOffset, 0);
+      lds_dma<16>(rs, lds_addr(wt + i * 512), lch * 8 < a.D ? row * (int)stride * 2 + lch * 16 : kPadOffset, 0);
     }
   };
   auto landed = [&]() {

@@ -332,6 +332,10 @@ __device__ __forceinline__ uint32_t lds_addr(lds_cptr p) { return (uint32_t)(uin
 // physical chunk p of a row fetches logical chunk p ^ swz(row).  Rows past the
 // end of the source are zero-filled by the buffer range check.  The loads are
 // asynchronous: call wait_all() before the barrier that publishes the tile.
+// Byte offset of a lane whose chunk lies beyond the tensor's head dim (head dims below the tile width run
+// zero-padded): past the end of every descriptor, so the range check fills the chunk with zeros.
+constexpr int kPadOffset = 0x7ffffff0;
+
 template <int HD, int ROWS, int NT>
 struct AsyncTileLoader {
   static constexpr int CH = HD / 8;            // 16-byte chunks per row
@@ -342,9 +346,6 @@ struct AsyncTileLoader {
   int row_in_pass;  // row of this lane within one pass over the tile
   int gchunk;       // logical chunk this lane fetches
   int wave;
-  // Byte offset of a lane whose chunk lies beyond the tensor's head dim (head dims below the tile width run
-  // zero-padded): past the end of every descriptor, so the range check fills the chunk with zeros.
-  static constexpr int kPadOffset = 0x7ffffff0;
 
   // `d`: head dim of the tensors, a multiple of 8 not above HD
   __device__ __forceinline__ void init(int tid, int d = HD) {
@@ -428,7 +429,7 @@ struct WaveTileLoader {
     for (int i = 0; i < N; i++) {
       const int row = i * RPW + prow;
       const int lch = pch ^ Tile<HD>::swz(row);
-      lds_dma<16>(rs, lds_addr(tile + i * 512), lch * 8 < d ? row * (int)stride_bytes + lch * 16 : 0x7ffffff0, 0);
+      lds_dma<16>(rs, lds_addr(tile + i * 512), lch * 8 < d ? row * (int)stride_bytes + lch * 16 : kPadOffset, 0);
     }
   }
   // at most K of this wave's vector-memory loads (the youngest) still in flight
