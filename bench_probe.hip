@@ -3,10 +3,12 @@
 // by its power limit and depends on the operand bits (zeros run near the nominal clock, random
 // operands several hundred MHz lower), so a roofline fraction against the nominal peak says little
 // without this number measured next to it on the same device with the same kind of data.
+//
+// Built into bench_probe.so beside bench.py, which is its only user; it is not part of libmoda_hip.so.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "tile.h"
+#include "moda_amd/csrc/tile.h"
 
 namespace moda {
 
@@ -40,11 +42,18 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(const i32x4* operands, 
   if (s == 12345.678f) sink[0] = s;  // keeps the loop alive; practically never true
 }
 
-hipError_t launch_mfma_probe(const void* operands, int64_t iters, uint64_t* clocks, float* sink, int blocks,
-                             hipStream_t stream) {
-  hipLaunchKernelGGL(mfma_probe_kernel, dim3((unsigned)blocks), dim3(512), 0, stream,
-                     reinterpret_cast<const i32x4*>(operands), iters, clocks, sink);
-  return hipGetLastError();
-}
-
 }  // namespace moda
+
+// Runs `iters` rounds of four independent bf16 MFMAs per wave (eight waves per workgroup, `workgroups`
+// workgroups; 32768 FLOP per MFMA) on the register operands found in `operands` (device memory, 512 x 16
+// bytes: lane l of operand j reads entry 64*j + l; entries 0..255 feed the A side, 256..511 the B side).
+// `clocks` (device, two uint64, may be NULL) receives the loop's duration in shader-clock cycles and in
+// 100 MHz ticks; `sink` is 4 bytes of device scratch.  Returns 0, -1 for bad arguments, -2 for a failed launch.
+extern "C" int bench_probe_mfma(const void* operands, int64_t iters, int64_t workgroups, uint64_t* clocks, float* sink,
+                                void* stream) {
+  if (!operands || !sink || iters < 0 || workgroups <= 0 || workgroups > (1 << 20)) return -1;
+  if ((uintptr_t)operands % 16 != 0) return -1;
+  hipLaunchKernelGGL(moda::mfma_probe_kernel, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream,
+                     reinterpret_cast<const moda::i32x4*>(operands), iters, clocks, sink);
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}

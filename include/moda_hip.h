@@ -46,7 +46,10 @@
  * the longest sequence.  Sequences attend only within themselves; chunks of
  * CHUNK_VISIBLE are counted from each sequence's first token.  The offsets are read on
  * the device only: the host cannot check them, rows outside [0, total_tokens) named by
- * them are out-of-bounds accesses.
+ * them are out-of-bounds accesses.  A caller that also has the offsets in host memory may pass them as
+ * cu_seqlens_host: they are then validated, and packed batches with head dims above 128 run on the matrix cores
+ * as one launch per sequence (the fixed-length 256-wide kernels on each sequence's rows; the result is the same
+ * as one call per sequence); without the host copy that combination runs on the vector-ALU kernels.
  */
 #ifndef MODA_HIP_H_
 #define MODA_HIP_H_
@@ -58,7 +61,7 @@
 extern "C" {
 #endif
 
-#define MODA_HIP_VERSION 104
+#define MODA_HIP_VERSION 105
 
 enum moda_hip_dtype { MODA_HIP_BF16 = 0, MODA_HIP_FP16 = 1, MODA_HIP_FP32 = 2 };
 
@@ -118,6 +121,8 @@ typedef struct moda_hip_desc {
   const int32_t* cu_seqlens; /* packed variable-length batch (see above): DEVICE array of B + 1 offsets, else NULL */
   int64_t total_tokens;      /* with cu_seqlens: cu_seqlens[B], the length of the packed token axis              */
   int64_t Dv;                /* head dim of v, vd, o, do, dv, dvd; 0 = D.  Dv != D runs on the vector-ALU kernels */
+  const int32_t* cu_seqlens_host; /* optional HOST copy of the B + 1 offsets of cu_seqlens (checked against T and
+                                     total_tokens), else NULL; see "Packed variable-length batch" above */
 } moda_hip_desc;
 
 /*
@@ -141,6 +146,8 @@ int moda_hip_fwd(const moda_hip_desc* desc, const void* q, const void* k, const 
  * summation order of dk, dv but nothing else.  Returns 0 for an invalid descriptor.
  */
 size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* desc);
+/* `workspace` below must be 4-byte aligned (MODA_HIP_EALIGN otherwise); the row segments are only used when it is
+ * 16-byte aligned as well. */
 
 /*
  * Backward.  Replaces parallel_moda_bwd and its kernels (moda_v14.py:1470-1842,
@@ -218,17 +225,12 @@ int moda_hip_depth_reorg_bwd(const void* d_cache, int64_t n_layers, int64_t slot
                              void* const* d_layers, void* stream);
 
 /*
- * Diagnostic, no counterpart in the reference: runs `iters` rounds of four independent bf16 MFMAs
- * per wave (eight waves per workgroup, `workgroups` workgroups; 32768 FLOP per MFMA) on the register
- * operands found in `operands` (device memory, 512 x 16 bytes: lane l of operand j reads entry
- * 64*j + l; entries 0..255 feed the A side, 256..511 the B side).  The matrix pipe of this GPU is
- * power limited and its sustained rate depends on the operand bits, so benchmarks time this call
- * with the same kind of data next to the attention kernels.  `clocks` (device, two uint64, may be
- * NULL) receives the loop's duration in shader-clock cycles and in 100 MHz ticks.  `sink` is 4 bytes
- * of device scratch.
+ * Which kernels a descriptor runs on: 1 = the matrix-core kernels (tensor rows must then be 16-byte aligned, see
+ * the top of this file), 0 = the vector-ALU kernels (element alignment), negative = the descriptor's error code.
+ * No counterpart in the reference; lets a host wrapper decide whether an input needs a contiguous copy without
+ * repeating the library's rule.  Touches no device.
  */
-int moda_hip_mfma_probe(const void* operands, int64_t iters, int64_t workgroups, uint64_t* clocks, float* sink,
-                        void* stream);
+int moda_hip_uses_matrix_cores(const moda_hip_desc* desc);
 
 /* Human-readable text for an error code (static storage). */
 const char* moda_hip_strerror(int code);

@@ -28,9 +28,9 @@ EXPORTS = (
     "moda_hip_bwd_static",
     "moda_hip_depth_reorg_fwd",
     "moda_hip_depth_reorg_bwd",
+    "moda_hip_uses_matrix_cores",
     "moda_hip_strerror",
     "moda_hip_version",
-    "moda_hip_mfma_probe",
 )
 
 
@@ -68,6 +68,7 @@ class Desc(Structure):
         ("cu_seqlens", c_void_p),
         ("total_tokens", c_int64),
         ("Dv", c_int64),
+        ("cu_seqlens_host", c_void_p),
     ]
 
 
@@ -106,10 +107,10 @@ def load():
     lib.moda_hip_depth_reorg_bwd.restype = c_int
     lib.moda_hip_depth_reorg_bwd.argtypes = [vp, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                              c_int32, POINTER(vp), vp]
+    lib.moda_hip_uses_matrix_cores.restype = c_int
+    lib.moda_hip_uses_matrix_cores.argtypes = [POINTER(Desc)]
     lib.moda_hip_strerror.restype = c_char_p
     lib.moda_hip_strerror.argtypes = [c_int]
-    lib.moda_hip_mfma_probe.restype = c_int
-    lib.moda_hip_mfma_probe.argtypes = [vp, c_int64, c_int64, vp, vp, vp]
     lib.moda_hip_version.restype = c_int
     lib.moda_hip_version.argtypes = []
     _lib = lib

@@ -23,6 +23,7 @@
 // registers: every output row has one writer, no atomics, no partial buffers.
 #include <type_traits>
 
+#include "geometry.h"
 #include "kargs.h"
 #include "tile.h"
 #include "tile16.h"
@@ -57,25 +58,15 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   const int ct = blockIdx.x / BHk;
   int b = bh / a_in.Hkv;
   const int hkv = bh % a_in.Hkv;
-  // the grid holds the sequence tiles of the longest sequence, then (when launched with them) the depth tiles
-  const int n_seq_tiles = a_in.has_seq ? (a_in.T + BN - 1) / BN : 0;
   SeqArgs<VARLEN> seq(a_in, b);
   const KArgs& a = seq.a;
   // sequence tiles come `nseg` workgroups each (row segments of one column tile are neighbours in the grid, the
   // heaviest column tile first), then the depth tiles
   const int nseg = SPLIT ? a.dkv_split : 1;
-  const bool dep = ct >= n_seq_tiles * nseg;
-  const int ncols = dep ? a.T * a.L : a.T;
-  const int seg = dep ? 0 : ct % nseg;
-  int tile = dep ? ct - n_seq_tiles * nseg : ct / nseg;
-  if (VARLEN && !dep && a.causal) {
-    // a causal sequence tile costs what lies behind it: count the grid's tiles from the end of the sequence, so
-    // that tiles of equal cost of all sequences are dispatched together, the heaviest of the whole batch first
-    tile -= n_seq_tiles - (a.T + BN - 1) / BN;
-    if (tile < 0) return;
-  }
-  const int c_first = tile * BN;
-  if (VARLEN && c_first >= ncols) return;  // a tile beyond this sequence of a variable-length batch
+  const ColTilePlan plan = col_tile_plan(a_in, a, ct, BN, BM, VARLEN, nseg);
+  if (VARLEN && !plan.active) return;  // a tile beyond this sequence of a variable-length batch
+  const bool dep = plan.dep;
+  const int ncols = plan.ncols, seg = plan.seg, c_first = plan.c_first;
   int c[NB];
   bool valid[NB], live[NB];  // live: a column with data (an unwritten depth slot is seen by no row: its K/V are
                            // replaced by zeros, its gradients come out zero)
@@ -110,33 +101,14 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   __builtin_amdgcn_s_waitcnt(0x0F70);
   asm volatile("" ::: "memory");
 
-  // visible query-row interval of a column
-  auto q_interval = [&](int col, int& lo, int& hi) {
-    if (!dep) {
-      lo = a.causal ? col * a.Gf : 0;
-      hi = a.Tq;
-    } else {
-      const int w = col / a.L;
-      lo = w * a.Gf;
-      hi = a.chunk ? min(a.T, (w / a.Cb + 1) * a.Cb) * a.Gf : (w + 1) * a.Gf;
-    }
-  };
+  // visible query-row interval of this lane's columns
   int qlo[NB], qhi[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     qlo[nb] = qhi[nb] = 0;
-    if (live[nb]) q_interval(c[nb], qlo[nb], qhi[nb]);
+    if (live[nb]) q_interval(a, dep, c[nb], qlo[nb], qhi[nb]);
   }
-  int wg_lo, wg_hi, tmp;
-  q_interval(c_first, wg_lo, tmp);
-  q_interval(min(ncols, c_first + BN) - 1, tmp, wg_hi);
-  int qt0 = wg_lo / BM;
-  int nqt = (wg_hi + BM - 1) / BM - qt0;
-  if (SPLIT && !dep) {  // this workgroup's share of the column tile's query tiles
-    const int lo = (int)((int64_t)nqt * seg / nseg), hi = (int)((int64_t)nqt * (seg + 1) / nseg);
-    qt0 += lo;
-    nqt = hi - lo;
-  }
+  const int qt0 = plan.qt0, nqt = plan.nqt;
   const int niter = nqt * a.hdiv;
 
   using Loader = AsyncTileLoader<HD, BM, 512>;
@@ -173,7 +145,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   uint32_t lds_q, lds_stat;
   auto prep = [&]() {
     if (f_left == 0) seek_head();
-    const uint32_t rows = (uint32_t)max(min(a.Tq - f_q0, BM), 0);  // only a head's top tile can be short
+    const uint32_t rows = (uint32_t)query_tile_rows(a, f_q0, BM);  // only a head's top tile can be short
     rs_q = rsrc_words(q_ptr, rows * q_row_bytes);
     rs_do = rsrc_words(do_ptr, rows * do_row_bytes);
     rs_stat = rsrc_words(st_ptr, rows > 0 ? (rows - 1) * stat_row_bytes + 4u : 0u);
@@ -770,11 +742,8 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   // depth columns: vector kernel, except in chunk-visible mode where a column has up to G*Cb visible rows
   const bool depth_by_columns = a.L > 0 && !a.chunk;
   const int64_t n_seq_tiles = a.has_seq ? (a.T + BN - 1) / BN : 0;
-  // chunk-visible depth columns: by whole chunks when a chunk's rows fit one query tile (tile widths up to 128:
-  // the chunk kernel's registers and LDS do not stretch to 256), else as column tiles
-  const bool depth_by_chunks = HD <= 128 && a.L > 0 && a.chunk && (int64_t)a.Cb * a.Gf <= 64;
-  const int64_t n_dep_tiles = (a.L > 0 && a.chunk && !depth_by_chunks) ? ((int64_t)a.T * a.L + BN - 1) / BN : 0;
-  const int64_t nblk = (n_seq_tiles * nseg + n_dep_tiles) * a.B * a.Hkv;
+  const bool depth_by_chunks = moda::depth_by_chunks(a, HD);
+  const int64_t nblk = col_kernel_blocks(a, HD, BN, nseg);
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   if (nblk > 0) {
     if (a.cu)

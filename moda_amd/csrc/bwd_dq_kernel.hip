@@ -14,6 +14,7 @@
 #include <algorithm>
 #include <type_traits>
 
+#include "geometry.h"
 #include "kargs.h"
 #include "tile.h"
 #include "tile16.h"
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   const KArgs& a = seq.a;
   const int Ld = NODEPTH ? 0 : a.L;  // depth slots per token
   const int nqt = (a.Tq + BM - 1) / BM;
-  const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
+  const int qt = query_tile_of(blockIdx.x, BH, BM, VARLEN ? a_in.Tq : a.Tq);
   if (VARLEN && qt >= nqt) return;
 
   i32x4 Qr[NB][KS], dOr[NB][KS];
@@ -93,43 +94,27 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     }
     lse[nb] = 0.f;
     delta[nb] = 0.f;
-    shi[nb] = dlo[nb] = dhi[nb] = 0;
     if (valid) {
       lse[nb] = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq];
       delta[nb] = a.delta[((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r];
-      const int t = r / a.Gf;
-      if (a.has_seq) shi[nb] = a.causal ? t + 1 : a.T;
-      if (Ld > 0) {
-        const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
-        dlo[nb] = lo_t * a.L;
-        dhi[nb] = a.chunk ? (t + 1) * a.L : dlo[nb] + a.Lv;
-      }
     }
+    const RowVis vis = row_visibility(a, r, Ld);
+    shi[nb] = vis.shi;
+    dlo[nb] = vis.dlo;
+    dhi[nb] = vis.dhi;
   }
   // the register operands must have arrived before the tile loads (issued behind the compiler's back) start
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt(0x0F70);
   asm volatile("" ::: "memory");
 
-  const int r_first = qt * BM;
-  const int r_last = min(a.Tq, r_first + BM) - 1;
-  const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
-  int n_seq = 0, n_full = 0;
-  if (a.has_seq) {
-    n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
-    n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
-  }
-  // Depth columns a wave alone can see (always outside chunk-visible mode, and in it when a chunk's rows fit a
-  // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span after the
-  // sequence tiles (see the end of the kernel).
-  constexpr bool OWN_FITS = Shape::W * 64 * HD * 2 <= 128 * 1024;  // one 32-column K and V tile per wave
-  const bool own_depth = OWN_FITS && Ld > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
-  int dep0 = 0, n_dep = 0;
-  if (Ld > 0 && !own_depth) {
-    const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
-    dep0 = lo_t * a.L;
-    n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
-  }
+  // Depth columns a wave alone can see are not streamed through the workgroup's ring: each wave fetches its own
+  // rows' span after the sequence tiles (see the end of the kernel), when a 32-column K and V tile per wave fit.
+  constexpr bool OWN_FITS = Shape::W * 64 * HD * 2 <= 128 * 1024;
+  const bool own_depth = OWN_FITS && waves_own_depth(a, Ld);
+  const RowTilePlan plan = row_tile_plan(a, qt, BM, BN, Ld > 0 && !own_depth);
+  int n_seq = plan.n_seq, n_full = plan.n_full, dep0 = plan.dep0;
+  const int n_dep = plan.n_dep;
   n_seq = __builtin_amdgcn_readfirstlane(n_seq);
   n_full = __builtin_amdgcn_readfirstlane(n_full);
   dep0 = __builtin_amdgcn_readfirstlane(dep0);
@@ -267,9 +252,9 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     lds_ptr Kt = smem + wv * (2 * 32 * HD), Vt = Kt + 32 * HD;
     const int rw0 = qt * BM + wv * WR;
     if (rw0 < a.Tq) {
-      const int tw0 = rw0 / a.Gf, tw1 = (min(a.Tq, rw0 + WR) - 1) / a.Gf;
-      const int c_beg = __builtin_amdgcn_readfirstlane((a.chunk ? (tw0 / a.Cb) * a.Cb : tw0) * a.L);
-      const int c_end = __builtin_amdgcn_readfirstlane((tw1 + 1) * a.L);
+      const DepthSpan span = own_depth_span(a, rw0, WR);
+      const int c_beg = __builtin_amdgcn_readfirstlane(span.c_beg);
+      const int c_end = __builtin_amdgcn_readfirstlane(span.c_end);
       const int nh = (c_end - c_beg + 31) / 32;
       const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
       const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
@@ -312,7 +297,7 @@ template <typename T, int HD>
 hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
   if (a.Tq == 0 || a.B * a.Hq == 0) return hipSuccess;
   constexpr int RPB = 256 / (HD / 8);
-  const int64_t nblk = (int64_t)((a.Tq + RPB - 1) / RPB) * a.B * a.Hq;
+  const int64_t nblk = delta_kernel_blocks(a, RPB);
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   hipLaunchKernelGGL((delta_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), 0, stream, a);
   return hipGetLastError();
@@ -327,7 +312,7 @@ hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dq_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;
   constexpr int rows = 16 * Shape::NB * Shape::W;
-  const int64_t nblk = (int64_t)((a.Tq + rows - 1) / rows) * a.B * a.Hq;
+  const int64_t nblk = row_kernel_blocks(a, rows);
   if (nblk == 0) return hipSuccess;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   hipLaunchKernelGGL((dq_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);

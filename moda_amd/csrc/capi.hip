@@ -12,8 +12,6 @@ namespace moda {
 hipError_t launch_fwd(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_delta(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_dq(const KArgs& a, int dtype, int hd, hipStream_t stream);
-hipError_t launch_mfma_probe(const void* operands, int64_t iters, uint64_t* clocks, float* sink, int blocks,
-                             hipStream_t stream);
 hipError_t launch_dkv(const KArgs& a, int dtype, int hd, hipStream_t stream);
 hipError_t launch_generic(const KArgs& a, int dtype, int D, int Dv, int which, hipStream_t stream);
 hipError_t launch_reorg(void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t n_tokens,
@@ -45,13 +43,17 @@ int value_dim(const moda_hip_desc* d) { return (int)(d->Dv > 0 ? d->Dv : d->D); 
 
 // The matrix-core kernels exist for tile widths 64, 128 and 256; any 16-bit head dim that is a multiple of 8 (whole
 // 16-byte chunks) up to 256 runs on the next width, zero-padded inside the kernels.
-// Packed variable-length batches with head dims above 128 stay on the vector-ALU kernels: the combination of the
-// 256-wide tiles, a packed batch and chunk-visible mode ended in a GPU memory fault whose cause has not been
-// found, so the whole packed + wide path is switched off until it is.
-bool use_mfma(const moda_hip_desc* d) {
+bool mfma_shape(const moda_hip_desc* d) {
   return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && d->D % 8 == 0 && d->D <= 256 &&
-         value_dim(d) == d->D && !(d->D > 128 && d->cu_seqlens);
+         value_dim(d) == d->D;
 }
+// Packed variable-length batches with head dims above 128 do not run the packed instantiations of the 256-wide
+// kernels: that combination (with chunk-visible mode) once ended in a GPU memory fault whose cause was never
+// found, so those instantiations stay switched off.  With a host copy of the offsets the batch runs as one launch
+// per sequence on the fixed-length 256-wide kernels (per_sequence below); without it, on the vector-ALU kernels.
+bool packed_wide(const moda_hip_desc* d) { return d->D > 128 && d->cu_seqlens; }
+bool per_sequence(const moda_hip_desc* d) { return mfma_shape(d) && packed_wide(d) && d->cu_seqlens_host; }
+bool use_mfma(const moda_hip_desc* d) { return mfma_shape(d) && !packed_wide(d); }
 int tile_width(const moda_hip_desc* d) { return d->D <= 64 ? 64 : d->D <= 128 ? 128 : 256; }
 
 // Validates the descriptor and fills the geometry part of KArgs.
@@ -99,8 +101,16 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
     if (d->total_tokens < d->T || ((uintptr_t)d->cu_seqlens % 4) != 0) return MODA_HIP_EINVAL;
     if (d->total_tokens * d->G >= (1ll << 30) || d->total_tokens * (d->L > 0 ? d->L : 1) >= (1ll << 30))
       return MODA_HIP_EUNSUPPORTED;
+    if (d->cu_seqlens_host) {  // the host copy can be checked: offsets start at 0, do not decrease, fit T and total
+      const int32_t* h = d->cu_seqlens_host;
+      if (h[0] != 0 || h[d->B] != d->total_tokens) return MODA_HIP_EINVAL;
+      for (int64_t i = 0; i < d->B; i++)
+        if (h[i + 1] < h[i] || h[i + 1] - h[i] > d->T) return MODA_HIP_EINVAL;
+    }
     a.cu = d->cu_seqlens;
     a.delta_pitch = (int)(plain ? d->total_tokens : d->total_tokens * d->G);
+  } else if (d->cu_seqlens_host) {
+    return MODA_HIP_EINVAL;
   }
   return MODA_HIP_OK;
 }
@@ -172,6 +182,32 @@ int static_workspace(void** out) {
   return MODA_HIP_OK;
 }
 
+
+// Sequence i of a packed batch as a fixed-length problem of batch size 1: the descriptor, and the element offsets
+// of its first query row, key row and depth row on the packed row axes.
+struct SeqView {
+  moda_hip_desc d;
+  int64_t q_row, k_row, d_row;
+};
+SeqView sequence_view(const moda_hip_desc* d, int64_t i) {
+  SeqView v;
+  v.d = *d;
+  const int64_t t0 = d->cu_seqlens_host[i];
+  v.d.B = 1;
+  v.d.T = d->cu_seqlens_host[i + 1] - t0;
+  v.d.cu_seqlens = nullptr;
+  v.d.cu_seqlens_host = nullptr;
+  v.d.total_tokens = 0;
+  v.q_row = d->mode == MODA_HIP_PLAIN_GQA ? t0 : t0 * d->G;
+  v.k_row = t0;
+  v.d_row = t0 * d->L;
+  return v;
+}
+const void* at(const void* p, int64_t row, int64_t stride, int esize) {
+  return p ? (const char*)p + row * stride * esize : nullptr;
+}
+void* at(void* p, int64_t row, int64_t stride, int esize) { return p ? (char*)p + row * stride * esize : nullptr; }
+
 #define MODA_REQ_PTR(p) \
   if (!(p)) return MODA_HIP_EINVAL
 #define MODA_REQ_ALIGN(p, s)                                    \
@@ -189,6 +225,18 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
   if (rc) return rc;
   if ((int64_t)a.B * a.Tq * a.Hq == 0) return MODA_HIP_OK;
   const int es = elem_size(d->dtype);
+  if (per_sequence(d)) {
+    MODA_REQ_PTR(lse);
+    for (int64_t i = 0; i < d->B; i++) {
+      const SeqView s = sequence_view(d, i);
+      if (s.d.T == 0) continue;
+      rc = moda_hip_fwd(&s.d, at(q, s.q_row, d->q.t, es), at(k, s.k_row, d->k.t, es), at(v, s.k_row, d->v.t, es),
+                        at(kd, s.d_row, d->kd.t, es), at(vd, s.d_row, d->vd.t, es), at(o, s.q_row, d->o.t, es),
+                        lse + s.q_row * a.Hq, stream);
+      if (rc) return rc;
+    }
+    return MODA_HIP_OK;
+  }
   const bool vec16 = use_mfma(d);
   MODA_REQ_PTR(q);
   MODA_REQ_PTR(o);
@@ -230,7 +278,7 @@ size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* d) {
   KArgs a;
   if (fill_geometry(d, a)) return 0;
   const size_t part = dkv_part_bytes(d, a, desired_dkv_split(d, a));
-  return part ? delta_bytes(a) + part : delta_bytes_exact(a);
+  return part ? delta_bytes(a) + part : delta_bytes_exact(a);  // packed batches: the row sums only
 }
 
 int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
@@ -263,6 +311,26 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
   if (rc) return rc;
   if (stages < 0 || stages > MODA_HIP_STAGE_ALL) return MODA_HIP_EINVAL;
   const int es = elem_size(d->dtype);
+  if (per_sequence(d) && (int64_t)a.B * a.Tq * a.Hq > 0) {
+    MODA_REQ_PTR(lse);
+    if (!workspace || workspace_bytes < delta_bytes_exact(a)) return MODA_HIP_EWORKSPACE;
+    for (int64_t i = 0; i < d->B; i++) {
+      const SeqView s = sequence_view(d, i);
+      if (s.d.T == 0) continue;
+      // every sequence keeps its own part of the row-sum workspace ([heads][its query rows]), so the stages of
+      // one backward may still be issued as separate calls
+      const size_t ws_off = (size_t)a.Hq * s.q_row * sizeof(float);
+      const size_t ws_len = (size_t)a.Hq * (d->mode == MODA_HIP_PLAIN_GQA ? s.d.T : s.d.T * d->G) * sizeof(float);
+      rc = moda_hip_bwd_stages(&s.d, at(q, s.q_row, d->q.t, es), at(k, s.k_row, d->k.t, es),
+                               at(v, s.k_row, d->v.t, es), at(kd, s.d_row, d->kd.t, es), at(vd, s.d_row, d->vd.t, es),
+                               at(o, s.q_row, d->o.t, es), lse + s.q_row * a.Hq, at(d_o, s.q_row, d->d_o.t, es),
+                               at(dq, s.q_row, d->dq.t, es), at(dk, s.k_row, d->dk.t, es), at(dv, s.k_row, d->dv.t, es),
+                               at(dkd, s.d_row, d->dkd.t, es), at(dvd, s.d_row, d->dvd.t, es),
+                               (char*)workspace + ws_off, ws_len, stages, stream);
+      if (rc) return rc;
+    }
+    return MODA_HIP_OK;
+  }
   const bool vec16 = use_mfma(d);
   const bool have_rows = (int64_t)a.B * a.Tq * a.Hq > 0;
   if (have_rows) {
@@ -296,10 +364,12 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
       MODA_REQ_ALIGN(dvd, d->dvd);
     }
     if (!workspace || workspace_bytes < delta_bytes_exact(a)) return MODA_HIP_EWORKSPACE;
+    if ((uintptr_t)workspace % sizeof(float) != 0) return MODA_HIP_EALIGN;
     // the row split of light launches uses what the workspace offers beyond the row sums: a caller that gives
     // less than moda_hip_bwd_workspace_bytes asks for (moda_hip_bwd_static) gets fewer segments or none
     int split = desired_dkv_split(d, a);
     while (split > 1 && delta_bytes(a) + dkv_part_bytes(d, a, split) > workspace_bytes) split /= 2;
+    if ((uintptr_t)workspace % 16 != 0) split = 1;  // the partial sums are written and read 16 bytes at a time
     a.dkv_split = split;
     a.dkv_part = (float*)((char*)workspace + delta_bytes(a));
   } else {
@@ -376,14 +446,11 @@ int moda_hip_depth_reorg_bwd(const void* d_cache, int64_t n_layers, int64_t slot
   return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
 }
 
-int moda_hip_mfma_probe(const void* operands, int64_t iters, int64_t workgroups, uint64_t* clocks, float* sink,
-                        void* stream) {
-  if (!operands || !sink || iters < 0 || workgroups <= 0 || workgroups > (1 << 20)) return MODA_HIP_EINVAL;
-  if ((uintptr_t)operands % 16 != 0) return MODA_HIP_EALIGN;
-  int rc = check_device();
+int moda_hip_uses_matrix_cores(const moda_hip_desc* d) {
+  KArgs a;
+  const int rc = fill_geometry(d, a);
   if (rc) return rc;
-  hipError_t e = moda::launch_mfma_probe(operands, iters, clocks, sink, (int)workgroups, (hipStream_t)stream);
-  return e == hipSuccess ? MODA_HIP_OK : MODA_HIP_ELAUNCH;
+  return (use_mfma(d) || per_sequence(d)) ? 1 : 0;
 }
 
 const char* moda_hip_strerror(int code) {

@@ -17,6 +17,7 @@
 #include <algorithm>
 #include <type_traits>
 
+#include "geometry.h"
 #include "kargs.h"
 #include "tile.h"
 #include "tile16.h"
@@ -53,10 +54,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   const KArgs& a = seq.a;
   const int Ld = NODEPTH ? 0 : a.L;  // depth slots per token
   const int nqt = (a.Tq + BM - 1) / BM;
-  // Heavy (late) tiles first.  In a variable-length batch the grid counts tiles from the end of the longest
-  // sequence, so that tiles of equal cost (equal row position) of all sequences are dispatched together and the
-  // heaviest of the whole batch first; the positions a shorter sequence does not have are dropped.
-  const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
+  // heavy (late) tiles first; the positions a shorter sequence of a variable-length batch does not have are dropped
+  const int qt = query_tile_of(blockIdx.x, BH, BM, VARLEN ? a_in.Tq : a.Tq);
   if (VARLEN && qt >= nqt) return;
   const int r = qt * BM + wave * 32 + n;
   const bool valid = r < a.Tq;
@@ -80,36 +79,14 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   asm volatile("" ::: "memory");
 
   // per-row visible column intervals [lo, hi) for the two phases
-  int shi = 0, dlo = 0, dhi = 0;
-  if (valid) {
-    if (a.has_seq) shi = a.causal ? t + 1 : a.T;
-    if (Ld > 0) {
-      const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
-      dlo = lo_t * a.L;
-      dhi = a.chunk ? (t + 1) * a.L : dlo + a.Lv;  // the token's filled slots
-    }
-  }
-  // workgroup column ranges
-  const int r_first = qt * BM;
-  const int r_last = min(a.Tq, r_first + BM) - 1;
-  const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
-  int n_seq = 0, n_full = 0;
-  if (a.has_seq) {
-    n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
-    // leading sequence tiles that every row of the workgroup sees completely (padding rows of the
-    // last workgroup compute on zero queries there and are never stored)
-    n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
-  }
-  // Depth columns a wave alone can see (always outside chunk-visible mode, and in it when a chunk's rows fit a
-  // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span after the
-  // sequence tiles (see the end of the kernel).
-  const bool own_depth = Ld > 0 && (!a.chunk || a.Cb * a.Gf <= 64);
-  int dep0 = 0, n_dep = 0;
-  if (Ld > 0 && !own_depth) {
-    const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
-    dep0 = lo_t * a.L;
-    n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
-  }
+  const RowVis vis = row_visibility(a, r, Ld);
+  const int shi = vis.shi, dlo = vis.dlo, dhi = vis.dhi;
+  // Depth columns a wave alone can see are not streamed through the workgroup's ring: each wave fetches its own
+  // rows' span after the sequence tiles (see the end of the kernel).
+  const bool own_depth = waves_own_depth(a, Ld);
+  const RowTilePlan plan = row_tile_plan(a, qt, BM, BN, Ld > 0 && !own_depth);
+  int n_seq = plan.n_seq, n_full = plan.n_full, dep0 = plan.dep0;
+  const int n_dep = plan.n_dep;
   // wave-uniform by construction, but computed with vector divisions: the explicit hint keeps the
   // loop control in scalar registers
   n_seq = __builtin_amdgcn_readfirstlane(n_seq);
@@ -357,9 +334,9 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
     lds_ptr Kt = smem + wv * (2 * 32 * HD), Vt = Kt + 32 * HD;
     const int rw0 = qt * BM + wv * 32;
     if (rw0 < a.Tq) {
-      const int tw0 = rw0 / a.Gf, tw1 = (min(a.Tq, rw0 + 32) - 1) / a.Gf;
-      const int c_beg = __builtin_amdgcn_readfirstlane((a.chunk ? (tw0 / a.Cb) * a.Cb : tw0) * a.L);
-      const int c_end = __builtin_amdgcn_readfirstlane((tw1 + 1) * a.L);
+      const DepthSpan span = own_depth_span(a, rw0, 32);
+      const int c_beg = __builtin_amdgcn_readfirstlane(span.c_beg);
+      const int c_end = __builtin_amdgcn_readfirstlane(span.c_end);
       const int nh = (c_end - c_beg + 31) / 32;
       const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
       const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
@@ -429,10 +406,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
   SeqArgs<VARLEN> seq(a_in, b);
   const KArgs& a = seq.a;
   const int nqt = (a.Tq + BM - 1) / BM;
-  // Heavy (late) tiles first.  In a variable-length batch the grid counts tiles from the end of the longest
-  // sequence, so that tiles of equal cost (equal row position) of all sequences are dispatched together and the
-  // heaviest of the whole batch first; the positions a shorter sequence does not have are dropped.
-  const int qt = (VARLEN ? (a_in.Tq + BM - 1) / BM : nqt) - 1 - blockIdx.x / BH;
+  // heavy (late) tiles first; the positions a shorter sequence of a variable-length batch does not have are dropped
+  const int qt = query_tile_of(blockIdx.x, BH, BM, VARLEN ? a_in.Tq : a.Tq);
   if (VARLEN && qt >= nqt) return;
   i32x4 Qr[NB][KS];
   int shi[NB], dlo[NB], dhi[NB];  // per-row visible column intervals [lo, hi) for the two phases
@@ -446,16 +421,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
       i32x4 z = {0, 0, 0, 0};
       Qr[nb][ks] = (valid && 32 * ks + 8 * q4 < a.D) ? *reinterpret_cast<const i32x4*>(qp + 32 * ks) : z;
     }
-    shi[nb] = dlo[nb] = dhi[nb] = 0;
-    if (valid) {
-      const int t = r / a.Gf;
-      if (a.has_seq) shi[nb] = a.causal ? t + 1 : a.T;
-      if (a.L > 0) {
-        const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
-        dlo[nb] = lo_t * a.L;
-        dhi[nb] = a.chunk ? (t + 1) * a.L : dlo[nb] + a.Lv;  // the token's filled slots
-      }
-    }
+    const RowVis vis = row_visibility(a, r, a.L);
+    shi[nb] = vis.shi;
+    dlo[nb] = vis.dlo;
+    dhi[nb] = vis.dhi;
   }
 
   // The register operands above must have arrived before the tile loads start: those are issued
@@ -465,23 +434,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
   __builtin_amdgcn_s_waitcnt(0x0F70);
   asm volatile("" ::: "memory");
 
-  // workgroup column ranges
-  const int r_first = qt * BM;
-  const int r_last = min(a.Tq, r_first + BM) - 1;
-  const int t_first = r_first / a.Gf, t_last = r_last / a.Gf;
-  int n_seq = 0, n_full = 0;
-  if (a.has_seq) {
-    n_seq = ((a.causal ? t_last + 1 : a.T) + BN - 1) / BN;
-    // leading sequence tiles that every row of the workgroup sees completely (padding rows of the
-    // last workgroup compute on zero queries there and are never stored)
-    n_full = min(n_seq, (a.causal ? t_first + 1 : a.T) / BN);
-  }
-  int dep0 = 0, n_dep = 0;
-  if (a.L > 0) {
-    const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
-    dep0 = lo_t * a.L;
-    n_dep = ((t_last + 1) * a.L - dep0 + BN - 1) / BN;
-  }
+  // the workgroup's column tiles: depth columns always stream through the ring here
+  const RowTilePlan plan = row_tile_plan(a, qt, BM, BN, a.L > 0);
+  int n_seq = plan.n_seq, n_full = plan.n_full, dep0 = plan.dep0;
+  const int n_dep = plan.n_dep;
   // wave-uniform by construction, but computed with vector divisions: the explicit hint keeps the
   // loop control in scalar registers
   n_seq = __builtin_amdgcn_readfirstlane(n_seq);
@@ -691,7 +647,7 @@ hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
   static LdsAttrState attr;
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;
-  const int64_t nblk = (int64_t)((a.Tq + 32 * Shape::W - 1) / (32 * Shape::W)) * a.B * a.Hq;
+  const int64_t nblk = row_kernel_blocks(a, 32 * Shape::W);
   if (nblk == 0) return hipSuccess;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   hipLaunchKernelGGL((fwd_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);
@@ -707,7 +663,7 @@ hipError_t launch_fwd_wide(const KArgs& a, hipStream_t stream) {
       allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_wide_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;
   constexpr int rows = 16 * Shape::NB * Shape::W;
-  const int64_t nblk = (int64_t)((a.Tq + rows - 1) / rows) * a.B * a.Hq;
+  const int64_t nblk = row_kernel_blocks(a, rows);
   if (nblk == 0) return hipSuccess;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
   hipLaunchKernelGGL((fwd_wide_kernel<T, HD, Shape, ADDR>), dim3((unsigned)nblk), dim3(64 * Shape::W), smem, stream, a);

@@ -44,7 +44,7 @@ struct KArgs {
 // sequence's length, so that the code after it addresses the sequence as batch 0 of a fixed-length problem.
 // The launch grid is sized for the longest sequence: callers drop the tiles beyond their own sequence.
 // `units`: 16-bit units per tensor element (the data pointers are typed for 16-bit elements).
-__device__ __forceinline__ void enter_sequence(KArgs& a, int& b, int units = 1) {
+__host__ __device__ __forceinline__ void enter_sequence(KArgs& a, int& b, int units = 1) {
   if (a.cu == nullptr) return;
   const int t0 = a.cu[b];
   const int T = a.cu[b + 1] - t0;

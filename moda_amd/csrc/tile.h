@@ -120,11 +120,11 @@ struct Tile {
   // chunks, bit 1 on top so that rows r and r + 2 of a four-row, four-chunk transposed read land in different
   // halves of the row.  (Measured with SQ_LDS_BANK_CONFLICT on all four operand read patterns: 0 for HD = 64,
   // 128 and 256; the first formula cut to three bits cost HD = 64 a second pass on every read.)
-  __device__ __forceinline__ static int swz(int row) {
+  __host__ __device__ __forceinline__ static int swz(int row) {
     return CH == 8 ? ((((row >> 1) & 1) << 2) | ((row >> 2) & 3)) : ((((row & 3) << 2) | ((row >> 2) & 3)) & (CH - 1));
   }
   // element offset of logical (row, chunk)
-  __device__ __forceinline__ static int off(int row, int chunk) { return row * HD + ((chunk ^ swz(row)) << 3); }
+  __host__ __device__ __forceinline__ static int off(int row, int chunk) { return row * HD + ((chunk ^ swz(row)) << 3); }
 };
 
 // Per-lane LDS offsets of the two operand read patterns, computed once.  Tile
@@ -287,6 +287,11 @@ inline hipError_t allow_dynamic_lds(LdsAttrState& state, const void* kernel, siz
 // flight.  Completion is the caller's business: s_waitcnt vmcnt via wait_all()/wait_but<>() and a
 // workgroup barrier before any wave reads the tile.  The compiler's own vmcnt waits stay correct
 // because vector-memory loads return in order and an unseen younger load only makes them stricter.
+// The compiler's hazard pass does not look inside inline assembly either: a vector-memory instruction
+// that reads a scalar register written by a vector-ALU instruction (v_readfirstlane, v_readlane of a
+// spilled scalar) fewer than five wait states earlier sees the register's OLD value.  The compiler places
+// such writes right in front of the block when scalar registers are short, so the block brings its own
+// wait states: s_mov (1) + s_nop 3 (4), which also covers the one wait state m0 needs.
 template <int BYTES>
 __device__ __forceinline__ void lds_dma(i32x4 rsrc, uint32_t lds_byte_addr, int voff, int soff) {
   static_assert(BYTES == 16 || BYTES == 4, "dwordx4 or dword");
@@ -302,12 +307,12 @@ __device__ __forceinline__ void lds_dma(i32x4 rsrc, uint32_t lds_byte_addr, int 
   rs[2] = __builtin_amdgcn_readfirstlane(rsrc[2]);
   rs[3] = __builtin_amdgcn_readfirstlane(rsrc[3]);
   if (BYTES == 16)
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
                  : "memory", "m0");
   else
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
                  : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
                  : "memory", "m0");
@@ -348,17 +353,24 @@ struct AsyncTileLoader {
   int wave;
 
   // `d`: head dim of the tensors, a multiple of 8 not above HD
-  __device__ __forceinline__ void init(int tid, int d = HD) {
+  __host__ __device__ __forceinline__ void init(int tid, int d = HD) {
     const int lane = tid & 63;
+#if defined(__HIP_DEVICE_COMPILE__)
     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#else
+    wave = tid >> 6;
+#endif
     row_in_pass = wave * RPW + lane / CH;
     gchunk = (lane % CH) ^ Tile<HD>::swz(row_in_pass);
     if (gchunk * 8 >= d) gchunk = -1;
   }
   // this lane's byte offset inside a tile whose rows are `stride_bytes` apart
-  __device__ __forceinline__ int lane_offset(int stride_bytes) const {
+  __host__ __device__ __forceinline__ int lane_offset(int stride_bytes) const {
     return gchunk < 0 ? kPadOffset : row_in_pass * stride_bytes + gchunk * 16;
   }
+  // the i-th of a wave's N loads of a tile: element offset of the 64 LDS slots it fills, tile rows it skips
+  __host__ __device__ __forceinline__ int lds_elems(int i) const { return (i * NW + wave) * 512; }
+  __host__ __device__ __forceinline__ static constexpr int rows_before(int i) { return i * NW * RPW; }
   // A source of rows: fixed descriptor over rows [row_base, row_end) of a (batch, head) slice whose
   // byte span fits 31 bits (kernels that may meet wider slices use load() below, which anchors a
   // descriptor at every tile at the price of 64-bit address arithmetic per tile).
@@ -369,7 +381,7 @@ struct AsyncTileLoader {
     int stride_bytes;
     int row_base;
   };
-  __device__ __forceinline__ Source source(const uint16_t* slice, int64_t row_stride, int row_base, int row_end) const {
+  __host__ __device__ __forceinline__ Source source(const uint16_t* slice, int64_t row_stride, int row_base, int row_end) const {
     Source s;
     s.stride_bytes = (int)row_stride * 2;
     s.row_base = row_base;
@@ -380,23 +392,28 @@ struct AsyncTileLoader {
     return s;
   }
   // rows [row0, row0 + ROWS) of the source into `tile`; rows past the source's end arrive as zeros
+  // scalar byte offset of load i of the tile that starts at row `row0` of the source
+  __host__ __device__ __forceinline__ static int source_soffset(const Source& s, int row0, int i) {
+    return (row0 - s.row_base + rows_before(i)) * s.stride_bytes;
+  }
   __device__ __forceinline__ void load_from(lds_ptr tile, const Source& s, int row0) const {
-    const int soff = (row0 - s.row_base) * s.stride_bytes;
     const i32x4 rs = rsrc_words(s.base, s.nbytes);
 #pragma unroll
-    for (int i = 0; i < N; i++)
-      lds_dma<16>(rs, lds_addr(tile + (i * NW + wave) * 512), s.voff, soff + i * NW * RPW * s.stride_bytes);
+    for (int i = 0; i < N; i++) lds_dma<16>(rs, lds_addr(tile + lds_elems(i)), s.voff, source_soffset(s, row0, i));
+  }
+  // bytes covered by the descriptor load() anchors at row `row0` of a slice that ends at row `row_end`
+  __host__ __device__ __forceinline__ static uint32_t anchored_bytes(int64_t row_stride, int row0, int row_end) {
+    const int rows_left = row_end - row0;
+    const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
+    return rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
   }
   __device__ __forceinline__ void load(lds_ptr tile, const uint16_t* src, int64_t row_stride, int row0,
                                        int row_end) const {
-    const int rows_left = row_end - row0;
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
-    const uint32_t nbytes = rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
-    const i32x4 rs = rsrc_words(src + (int64_t)row0 * row_stride, nbytes);
+    const i32x4 rs = rsrc_words(src + (int64_t)row0 * row_stride, anchored_bytes(row_stride, row0, row_end));
     const int voff = lane_offset((int)stride_bytes);
 #pragma unroll
-    for (int i = 0; i < N; i++)
-      lds_dma<16>(rs, lds_addr(tile + (i * NW + wave) * 512), voff, i * NW * RPW * (int)stride_bytes);
+    for (int i = 0; i < N; i++) lds_dma<16>(rs, lds_addr(tile + lds_elems(i)), voff, rows_before(i) * (int)stride_bytes);
   }
   // s_waitcnt vmcnt(0): every outstanding vector-memory load of this wave has landed
   __device__ __forceinline__ static void wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -415,10 +432,16 @@ template <int HD>
 struct WaveTileLoader {
   static constexpr int CH = HD / 8, RPW = 64 / CH, N = 32 / RPW;  // chunks per row, rows per load, loads per tile
   int prow, pch, d;
-  __device__ __forceinline__ void init(int lane, int head_dim) {
+  __host__ __device__ __forceinline__ void init(int lane, int head_dim) {
     prow = lane / CH;
     pch = lane % CH;
     d = head_dim;
+  }
+  // this lane's byte offset in load i of a tile (rows `stride_bytes` apart): its tile row is i * RPW + prow
+  __host__ __device__ __forceinline__ int lane_offset(int i, int stride_bytes) const {
+    const int row = i * RPW + prow;
+    const int lch = pch ^ Tile<HD>::swz(row);
+    return lch * 8 < d ? row * stride_bytes + lch * 16 : kPadOffset;
   }
   // rows [row0, row0 + nrows) of the slice at `base` (nrows <= 32; the rest of the tile arrives as zeros)
   __device__ __forceinline__ void fetch(lds_ptr tile, const uint16_t* base, int64_t row_stride, int64_t row0,
@@ -426,11 +449,7 @@ struct WaveTileLoader {
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const i32x4 rs = rsrc_words(base + row0 * row_stride, nrows > 0 ? (uint32_t)nrows * stride_bytes : 0u);
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-      const int row = i * RPW + prow;
-      const int lch = pch ^ Tile<HD>::swz(row);
-      lds_dma<16>(rs, lds_addr(tile + i * 512), lch * 8 < d ? row * (int)stride_bytes + lch * 16 : kPadOffset, 0);
-    }
+    for (int i = 0; i < N; i++) lds_dma<16>(rs, lds_addr(tile + i * 512), lane_offset(i, (int)stride_bytes), 0);
   }
   // at most K of this wave's vector-memory loads (the youngest) still in flight
   template <int K>

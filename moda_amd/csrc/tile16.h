@@ -41,7 +41,7 @@ __device__ __forceinline__ f32x4 mfma16<FP16>(i32x4 a, i32x4 b, f32x4 c) {
 }
 
 // First tile row (within a 16-row block) of the four that lane group q holds in an accumulator block.
-__device__ __forceinline__ constexpr int slot_base(int q) { return (0x4C80 >> (4 * q)) & 15; }
+__host__ __device__ __forceinline__ constexpr int slot_base(int q) { return (0x4C80 >> (4 * q)) & 15; }
 
 // Two accumulator blocks (rows 4q+i of each) -> the eight k slots of a B operand, rounded to 16 bits.
 template <typename T>

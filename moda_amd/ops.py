@@ -38,6 +38,8 @@ class PackedBatch(NamedTuple):
     n: int            # sequences
     max_len: int      # base tokens of the longest sequence
     total: int        # base tokens in the packed axis
+    host: object = None  # ctypes int32 array [n + 1]: the offsets again, in host memory (the library checks them and
+                         # can launch per sequence where it has no packed kernel)
 
 
 def _packed(cu_seqlens, q: torch.Tensor, rows_per_token: int) -> Optional[PackedBatch]:
@@ -60,7 +62,8 @@ def _packed(cu_seqlens, q: torch.Tensor, rows_per_token: int) -> Optional[Packed
         f"cu_seqlens ends at {total} base tokens but q holds {q.shape[1]} rows "
         f"({rows_per_token} per token)")
     cu = cu_seqlens.detach().to(device=q.device, dtype=torch.int32).contiguous()
-    return PackedBatch(cu, int(lens.numel()), int(lens.max()) if lens.numel() else 0, total)
+    host_arr = (ctypes.c_int32 * host.numel())(*host.tolist())
+    return PackedBatch(cu, int(lens.numel()), int(lens.max()) if lens.numel() else 0, total, host_arr)
 
 
 def _ptr(x: Optional[torch.Tensor]):
@@ -93,11 +96,28 @@ def _usable(x: Optional[torch.Tensor], vec16: bool = True) -> Optional[torch.Ten
     return x if ok else x.contiguous()
 
 
-def _matrix_core_path(q: torch.Tensor, val: torch.Tensor) -> bool:
-    """Whether the call runs on the matrix-core kernels (16-bit, head dim a multiple of 8 up to 256, the same for
-    keys and values)."""
-    return (q.dtype in (torch.bfloat16, torch.float16) and q.shape[3] % 8 == 0 and q.shape[3] <= 256
-            and val.shape[3] == q.shape[3])
+def _matrix_core_path(q: torch.Tensor, val: torch.Tensor, packed: Optional["PackedBatch"] = None) -> bool:
+    """Whether the call runs on the matrix-core kernels, whose rows must be 16-byte aligned.  The rule is the
+    library's own (``moda_hip_uses_matrix_cores``): it is asked with a descriptor that carries what the rule reads
+    -- dtype, head dims, whether the batch is packed and has host offsets."""
+    if q.dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {q.dtype}; expected bf16, fp16 or fp32")
+    d = Desc()
+    d.struct_size = ctypes.sizeof(Desc)
+    d.dtype = _DTYPES[q.dtype]
+    d.mode = _lib.NONCAUSAL
+    d.B = d.T = d.H = d.G = 1
+    d.D, d.Dv = q.shape[3], val.shape[3]
+    d.scale = 1.0
+    if packed is not None:
+        d.B, d.T, d.total_tokens = packed.n, packed.max_len, packed.total
+        d.cu_seqlens = packed.cu.data_ptr()
+        if packed.host is not None:
+            d.cu_seqlens_host = ctypes.cast(packed.host, ctypes.c_void_p)
+    rc = _lib.load().moda_hip_uses_matrix_cores(ctypes.byref(d))
+    if rc < 0:  # a head dim the library rejects: the launch itself will report it
+        return False
+    return rc == 1
 
 
 def _strides(x: Optional[torch.Tensor]) -> Strides:
@@ -140,6 +160,8 @@ def _desc(mode, q, k, v, kd, vd, G, L, chunk_tokens, scale, o=None, do=None, dq=
         d.B, d.T = packed.n, packed.max_len
         d.cu_seqlens = packed.cu.data_ptr()
         d.total_tokens = packed.total
+        if packed.host is not None:
+            d.cu_seqlens_host = ctypes.cast(packed.host, ctypes.c_void_p)
     d.chunk_tokens = chunk_tokens
     d.flags = _lib.FLAG_ACCUMULATE_DEPTH_GRADS if accumulate_depth else 0
     d.scale = float(scale)
@@ -214,7 +236,7 @@ def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None, 
     _check_shapes(mode, q, k, v, kd, vd, G)
     _check_device(q)
     _same_dtype(q, k, v, kd, vd)
-    vec16 = _matrix_core_path(q, vd if mode == _lib.DEPTH_ONLY else v)
+    vec16 = _matrix_core_path(q, vd if mode == _lib.DEPTH_ONLY else v, packed)
     q, k, v, kd, vd = (_usable(x, vec16) for x in (q, k, v, kd, vd))
     src = kd if mode == _lib.DEPTH_ONLY else k
     T = q.shape[1] // G if mode == _lib.DEPTH_ONLY else k.shape[1]
@@ -247,7 +269,7 @@ def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages
     _check_shapes(mode, q, k, v, kd, vd, G, o=o, do=do, lse=lse)
     _check_device(q)
     _same_dtype(q, k, v, kd, vd, o, do)
-    vec16 = _matrix_core_path(q, vd if mode == _lib.DEPTH_ONLY else v)
+    vec16 = _matrix_core_path(q, vd if mode == _lib.DEPTH_ONLY else v, packed)
     q, k, v, kd, vd, o, do = (_usable(x, vec16) for x in (q, k, v, kd, vd, o, do))
     lse = lse.contiguous()
     T = q.shape[1] // G if mode == _lib.DEPTH_ONLY else k.shape[1]
@@ -463,8 +485,11 @@ def parallel_moda(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_
 # ---------------------------------------------------------------------------
 # chunk-visible MoDA -- moda_v16.py
 # ---------------------------------------------------------------------------
-def _chunk_tokens(moda_group_num: int, customized_BT: Optional[int]) -> int:
-    rows = customized_BT if customized_BT is not None else DEFAULT_CHUNK_ROWS
+def _chunk_tokens(moda_group_num: int, chunk_rows: Optional[int]) -> int:
+    """Base tokens per chunk.  The reference's launchers take ``customized_BT`` but overwrite it with 64 rows on
+    every device (moda_v16.py:545-584), so a chunk is always 64 query rows there; ``chunk_rows`` (an argument
+    the reference does not have) is the way to ask for another chunk size here."""
+    rows = chunk_rows if chunk_rows is not None else DEFAULT_CHUNK_ROWS
     assert (
         rows % moda_group_num == 0
     ), "BT must be divisible by moda_group_num to keep chunk-visible base_t aligned"
@@ -473,11 +498,12 @@ def _chunk_tokens(moda_group_num: int, customized_BT: Optional[int]) -> int:
 
 def parallel_moda_chunk_visible_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, cached_v=None,
                                     moda_group_num=1, customized_BT=None, customized_BS=None, customized_BK=None,
-                                    customized_BV=None, customized_num_warps=None):
-    """moda_v16.py:498-633.  ``customized_BT`` is the chunk size in query rows (default 64)."""
+                                    customized_BV=None, customized_num_warps=None, chunk_rows=None):
+    """moda_v16.py:498-633.  The tile-size knobs are accepted and ignored, ``customized_BT`` included (the
+    reference overwrites it with 64, moda_v16.py:581-585); ``chunk_rows`` sets the chunk size in query rows."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
     assert q.shape[2] == k.shape[2], "Implicit head-dimension GQA is not allowed."
-    cb = _chunk_tokens(moda_group_num, customized_BT)
+    cb = _chunk_tokens(moda_group_num, chunk_rows)
     return _raw_fwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, scale, moda_group_num, cb,
                     packed=_packed(cu_seqlens, q, moda_group_num))
 
@@ -485,12 +511,12 @@ def parallel_moda_chunk_visible_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, c
 def parallel_moda_chunk_visible_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None,
                                     cached_k=None, cached_v=None, moda_group_num=1, customized_BT=None,
                                     customized_BS=None, customized_BK=None, customized_BV=None,
-                                    customized_num_warps=None):
-    """moda_v16.py:2099-2343."""
+                                    customized_num_warps=None, chunk_rows=None):
+    """moda_v16.py:2099-2343 (``customized_BT`` ignored as there, ``chunk_rows`` as in the forward)."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
     if scale is None:
         scale = q.shape[-1] ** -0.5
-    cb = _chunk_tokens(moda_group_num, customized_BT)
+    cb = _chunk_tokens(moda_group_num, chunk_rows)
     dq, dk, dv, dkd, dvd = _raw_bwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, o, lse, do, scale,
                                     moda_group_num, cb, packed=_packed(cu_seqlens, q, moda_group_num))
     return dq, dk, dv, None, dkd, dvd
@@ -502,9 +528,9 @@ class ParallelMixtureOfDepthAttentionChunkVisibleFunction(torch.autograd.Functio
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, q, k, v, g, scale, cu_seqlens, cached_k=None, cached_v=None, moda_group_num=1,
-                customized_BT=None):
+                chunk_rows=None):
         o, lse = _autograd_forward(ctx, parallel_moda_chunk_visible_fwd, q, k, v, g, scale, cu_seqlens, cached_k,
-                                   cached_v, moda_group_num, customized_BT=customized_BT)
+                                   cached_v, moda_group_num, chunk_rows=chunk_rows)
         ctx.mark_non_differentiable(lse)
         return o, lse
 
@@ -518,16 +544,17 @@ class ParallelMixtureOfDepthAttentionChunkVisibleFunction(torch.autograd.Functio
 def parallel_moda_chunk_visible(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_seqlens=None,
                                 moda_group_num=1, head_first=False, need_lse=False, return_depth_grads=True,
                                 warn_shape=True, customized_BT=None, customized_BS=None, customized_BT_backward=None,
-                                customized_BS_backward=None):
-    """Chunk-visible MoDA; signature of moda_v16.py:3614-3632.  A query of base
-    token ``t`` additionally sees the depth slots of tokens
-    ``floor(t/Cb)*Cb .. t`` with ``Cb = customized_BT // moda_group_num``
-    (``customized_BT`` defaults to 64 query rows)."""
+                                customized_BS_backward=None, chunk_rows=None):
+    """Chunk-visible MoDA; signature of moda_v16.py:3614-3632 plus ``chunk_rows``.  A query of base
+    token ``t`` additionally sees the depth slots of tokens ``floor(t/Cb)*Cb .. t`` with
+    ``Cb = 64 // moda_group_num``.  The four ``customized_*`` arguments are accepted and dropped exactly as the
+    reference's wrapper drops them (moda_v16.py:3646-3650: a chunk is 64 query rows whatever they say);
+    ``chunk_rows``, which the reference does not have, selects another chunk size in query rows."""
     q, k, v, g, cached_k, cached_v, scale = _prepare_inputs(
         "parallel_moda_chunk_visible", q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first,
         return_depth_grads, warn_shape)
     o, lse = ParallelMixtureOfDepthAttentionChunkVisibleFunction.apply(
-        q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, customized_BT)
+        q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, chunk_rows)
     return (o, lse) if need_lse else o
 
 

@@ -32,8 +32,8 @@ def test_descriptor_layout_and_version():
     from moda_amd import _lib
 
     lib = _lib.load()
-    assert lib.moda_hip_version() == 104
-    assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24 + 24
+    assert lib.moda_hip_version() == 105
+    assert ctypes.sizeof(_lib.Desc) == 16 + 7 * 8 + 8 + 12 * 24 + 24 + 8
     assert _lib.Desc.cu_seqlens.offset == 80 + 12 * 24
     assert _lib.Desc.q.offset == 80
     # a descriptor with the wrong struct_size is rejected without touching any device
@@ -91,6 +91,114 @@ def test_descriptor_validation_codes():
     arr = (ctypes.c_void_p * 1)(0x1000)
     assert lib.moda_hip_depth_reorg_fwd(arr, 1, 3, 3, 1, 4, 1, 64, _lib.BF16, ok, null) == -1  # slot out of range
     assert lib.moda_hip_depth_reorg_fwd(arr, 0, 0, 3, 1, 4, 1, 64, _lib.BF16, ok, null) == 0   # nothing to do
+
+
+def test_matrix_core_routing_rule_is_the_librarys():
+    """The host wrapper asks the library which kernels a call runs on (rows must be 16-byte aligned for the
+    matrix kernels): every combination of dtype, head dims and packing, against the rule stated in the header."""
+    from moda_amd import _lib, ops
+
+    lib = _lib.load()
+    host = (ctypes.c_int32 * 3)(0, 5, 13)
+    for dtype, tdt in ((_lib.BF16, torch.bfloat16), (_lib.FP16, torch.float16), (_lib.FP32, torch.float32)):
+        for D in (8, 36, 64, 100, 128, 136, 192, 256):
+            for Dv in (D, 64 if D != 64 else 32):
+                for packed in (None, "device_only", "with_host"):
+                    d = _lib.Desc()
+                    d.struct_size = ctypes.sizeof(_lib.Desc)
+                    d.dtype, d.mode = dtype, _lib.CAUSAL
+                    d.B, d.T, d.H, d.G, d.D, d.Dv, d.L = 1, 8, 1, 1, D, Dv, 0
+                    d.scale = 1.0
+                    pb = None
+                    if packed:
+                        d.B, d.T, d.total_tokens, d.cu_seqlens = 2, 8, 13, 0x1000
+                        cu = torch.tensor([0, 5, 13], dtype=torch.int32)
+                        pb = ops.PackedBatch(cu, 2, 8, 13, host if packed == "with_host" else None)
+                        if packed == "with_host":
+                            d.cu_seqlens_host = ctypes.cast(host, ctypes.c_void_p)
+                    want = dtype != _lib.FP32 and D % 8 == 0 and Dv == D and not (D > 128 and packed == "device_only")
+                    assert lib.moda_hip_uses_matrix_cores(ctypes.byref(d)) == int(want), (dtype, D, Dv, packed)
+                    q, v = torch.zeros(1, 8, 1, D, dtype=tdt), torch.zeros(1, 8, 1, Dv, dtype=tdt)
+                    assert ops._matrix_core_path(q, v, pb) == want, (dtype, D, Dv, packed)
+    bad = _lib.Desc()
+    bad.struct_size = 4
+    assert lib.moda_hip_uses_matrix_cores(ctypes.byref(bad)) == -1
+
+
+def test_host_offsets_are_validated():
+    from moda_amd import _lib
+
+    lib = _lib.load()
+
+    def desc(offsets, T, total, with_device=True):
+        d = _lib.Desc()
+        d.struct_size = ctypes.sizeof(_lib.Desc)
+        d.dtype, d.mode = _lib.BF16, _lib.CAUSAL
+        d.B, d.T, d.H, d.G, d.D, d.L = len(offsets) - 1, T, 1, 1, 64, 0
+        d.scale = 1.0
+        d.total_tokens = total
+        if with_device:
+            d.cu_seqlens = 0x1000
+        arr = (ctypes.c_int32 * len(offsets))(*offsets)
+        d.cu_seqlens_host = ctypes.cast(arr, ctypes.c_void_p)
+        return d, arr
+
+    d, keep = desc([0, 5, 13], 8, 13)
+    assert lib.moda_hip_bwd_workspace_bytes(ctypes.byref(d)) == 13 * 4
+    for offsets, T, total in (([1, 5, 13], 8, 13),   # does not start at 0
+                              ([0, 9, 5, 13], 9, 13),  # decreases
+                              ([0, 5, 12], 8, 13),    # does not end at total_tokens
+                              ([0, 4, 13], 8, 13)):   # a sequence longer than T
+        d, keep = desc(offsets, T, total)
+        assert lib.moda_hip_uses_matrix_cores(ctypes.byref(d)) == -1, offsets
+    d, keep = desc([0, 5, 13], 8, 13, with_device=False)  # host offsets without the device array
+    assert lib.moda_hip_uses_matrix_cores(ctypes.byref(d)) == -1
+
+
+def test_workspace_alignment_codes():
+    from moda_amd import _lib
+
+    lib = _lib.load()
+    d = _lib.Desc()
+    d.struct_size = ctypes.sizeof(_lib.Desc)
+    d.dtype, d.mode = _lib.BF16, _lib.CAUSAL
+    d.B, d.T, d.H, d.G, d.D, d.L = 1, 8, 1, 1, 64, 0
+    d.scale = 1.0
+    for f in ("q", "k", "v", "o", "d_o", "dq", "dk", "dv"):
+        getattr(d, f).b, getattr(d, f).t, getattr(d, f).h = 512, 64, 64
+    ok = ctypes.c_void_p(0x1000)
+    args = [ok] * 3 + [None, None] + [ok] * 6 + [None, None]
+    # a workspace pointer that is not 4-byte aligned is refused before anything is launched or dereferenced
+    assert lib.moda_hip_bwd(ctypes.byref(d), *args, ctypes.c_void_p(0x1002), 64, None) == -3
+    assert lib.moda_hip_bwd(ctypes.byref(d), *args, None, 64, None) == -4
+    assert lib.moda_hip_bwd(ctypes.byref(d), *args, ok, 8, None) == -4
+
+
+def test_import_shim_names_and_reference_loops():
+    import os
+    import sys
+
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "moda_amd", "compat")
+    sys.path.insert(0, root)
+    try:
+        for m in [m for m in sys.modules if m == "fla" or m.startswith("fla.")]:
+            del sys.modules[m]
+        import fla.ops.moda as shim
+        import moda_amd
+
+        assert shim.parallel_moda is moda_amd.parallel_moda
+        assert shim.parallel_moda_chunk_visible_bwd is moda_amd.parallel_moda_chunk_visible_bwd
+        # the reference package also exports its torch loops; here that is an ImportError that says where to look
+        with pytest.raises(ImportError, match="oracle/moda_oracle.py"):
+            from fla.ops.moda import naive_mixture_of_depth_causal_ref  # noqa: F401
+        with pytest.raises(ImportError, match="reference's torch loops"):
+            shim.naive_mixture_of_depth_causal_chunk_visible_ref
+        with pytest.raises(AttributeError):
+            shim.no_such_name
+    finally:
+        sys.path.remove(root)
+        for m in [m for m in sys.modules if m == "fla" or m.startswith("fla.")]:
+            del sys.modules[m]
 
 
 def test_missing_library_fails_loudly(monkeypatch):
