@@ -33,8 +33,11 @@
  * with 0 < L_valid < L the depth tensors keep their L slots per token but only
  * slots l < L_valid are visible; results equal those for the compacted tensors
  * [B, T*L_valid, H, D], and dkd, dvd are written as zeros in the other slots.
- * The invisible slots are still read (and multiplied by zero): they must hold
- * finite values.  Not available with MODA_HIP_CHUNK_VISIBLE.
+ * The invisible slots of kd, vd are never read: they may hold anything, bit patterns of
+ * NaN or Inf included (an uninitialised cache).  Every mode with a depth stream takes it.
+ * On the matrix-core kernels the rows of 64 / L_valid + 2 tokens of a depth tensor
+ * ((64 / L_valid + 2) * L * row stride bytes) must span less than 2 GiB
+ * (MODA_HIP_EUNSUPPORTED otherwise).
  *
  * Packed variable-length batch (the reference carries a cu_seqlens argument but asserts
  * it away, moda_v14.py:83-101, 2672-2673): with cu_seqlens != NULL the tensors have no
@@ -92,7 +95,7 @@ enum moda_hip_flag {
    * backward of layer n (L_valid = n) then adds its share to slots < n, and a layer's K/V gradient is
    * a slice of that buffer: no per-layer rebuild of the cache and no scatter of its gradient
    * (vision_tasks/deit/models.py:361-390 does both for every layer).  Still one writer per row and
-   * no atomics.  Not available with MODA_HIP_CHUNK_VISIBLE.
+   * no atomics.  Every mode with a depth stream takes it.
    */
   MODA_HIP_FLAG_ACCUMULATE_DEPTH_GRADS = 1
 };

@@ -23,6 +23,9 @@
 // registers: every output row has one writer, no atomics, no partial buffers.
 #include <type_traits>
 
+// the tile loads of this file's kernels keep five wait states from vector-ALU writes of their scalar operands in
+// the compiled code (checked by tests/test_inline_asm_hazards_cpu.py): no padding inside the load blocks
+#define MODA_DMA_NOP 0
 #include "geometry.h"
 #include "kargs.h"
 #include "tile.h"
@@ -68,14 +71,15 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   const bool dep = plan.dep;
   const int ncols = plan.ncols, seg = plan.seg, c_first = plan.c_first;
   int c[NB];
-  bool valid[NB], live[NB];  // live: a column with data (an unwritten depth slot is seen by no row: its K/V are
-                           // replaced by zeros, its gradients come out zero)
+  bool valid[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     c[nb] = c_first + kblk * (16 * NB) + 16 * nb + n;
     valid[nb] = c[nb] < ncols;
-    live[nb] = valid[nb] && !(dep && (c[nb] % a.L) >= a.Lv);
   }
+  // the column's row in its tensor: the key's row, or the depth slot's (depth columns are counted on the compact
+  // axis of the slots that hold data); computed where it is used, at both ends of the kernel, not kept in between
+  auto column_row = [&](int nb) -> int64_t { return dep ? depth_row_of(a, c[nb]) : (int64_t)c[nb]; };
 
   // stationary operand of this wave's role: K rows (A) or V rows (B)
   i32x4 Sr[NB][KS];
@@ -84,14 +88,16 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
                                  : (dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h);
     const int64_t st = role_b ? (dep ? a.svd.t : a.sv.t) : (dep ? a.skd.t : a.sk.t);
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++)
+    for (int nb = 0; nb < NB; nb++) {
+      const int64_t crow = column_row(nb);
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         i32x4 z = {0, 0, 0, 0};
-        Sr[nb][ks] = (live[nb] && 32 * ks + 8 * q4 < a.D)
-                         ? *reinterpret_cast<const i32x4*>(src + (int64_t)c[nb] * st + 32 * ks + 8 * q4)
+        Sr[nb][ks] = (valid[nb] && 32 * ks + 8 * q4 < a.D)
+                         ? *reinterpret_cast<const i32x4*>(src + crow * st + 32 * ks + 8 * q4)
                          : z;
       }
+    }
   }
 
   // The register operands above must have arrived before the tile loads start: those are issued
@@ -106,7 +112,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     qlo[nb] = qhi[nb] = 0;
-    if (live[nb]) q_interval(a, dep, c[nb], qlo[nb], qhi[nb]);
+    if (valid[nb]) q_interval(a, dep, c[nb], qlo[nb], qhi[nb]);
   }
   const int qt0 = plan.qt0, nqt = plan.nqt;
   const int niter = nqt * a.hdiv;
@@ -378,21 +384,42 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
     if (valid[nb]) {
       uint16_t* outp;
       float mul;
+      const int64_t crow = column_row(nb);
       if (!role_b) {  // dV
-        outp = dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)c[nb] * a.sdvd.t
-                   : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c[nb] * a.sdv.t;
+        outp = dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + crow * a.sdvd.t
+                   : a.dv + b * a.sdv.b + hkv * a.sdv.h + crow * a.sdv.t;
         mul = 1.f;
       } else {  // dK
-        outp = dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)c[nb] * a.sdkd.t
-                   : a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c[nb] * a.sdk.t;
+        outp = dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + crow * a.sdkd.t
+                   : a.dk + b * a.sdk.b + hkv * a.sdk.h + crow * a.sdk.t;
         mul = a.scale;
       }
+      if (dep && a.accum_depth) {
+        // add to what the row holds (this lane is its only writer).  One 8-byte piece at a time, in order: with the
+        // old values of all pieces fetched up front the kernel would not fit its registers
 #pragma unroll
-      for (int d = 0; d < MB; d++) {
-        i32x2 w;
-        w[0] = pack2<T>(acc[d][nb][0] * mul, acc[d][nb][1] * mul);
-        w[1] = pack2<T>(acc[d][nb][2] * mul, acc[d][nb][3] * mul);
-        if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(outp + 16 * d + 4 * q4) = w;
+        for (int d = 0; d < MB; d++) {
+          if (16 * d + 4 * q4 < a.D) {
+            i32x2* dst = reinterpret_cast<i32x2*>(outp + 16 * d + 4 * q4);
+            const i32x2 old = *dst;
+            float o0, o1, o2, o3;
+            unpack2<T>(old[0], o0, o1);
+            unpack2<T>(old[1], o2, o3);
+            i32x2 w;
+            w[0] = pack2<T>(acc[d][nb][0] * mul + o0, acc[d][nb][1] * mul + o1);
+            w[1] = pack2<T>(acc[d][nb][2] * mul + o2, acc[d][nb][3] * mul + o3);
+            *dst = w;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int d = 0; d < MB; d++) {
+          i32x2 w;
+          w[0] = pack2<T>(acc[d][nb][0] * mul, acc[d][nb][1] * mul);
+          w[1] = pack2<T>(acc[d][nb][2] * mul, acc[d][nb][3] * mul);
+          if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(outp + 16 * d + 4 * q4) = w;
+        }
       }
     }
 }
@@ -448,20 +475,19 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
   const float sc = a.scale * kLog2e;
   OperandAddr<HD> oa;
   oa.init(lane);
-  const int c_end = t1 * a.L;
+  const int c_end = t1 * a.Lv;  // depth columns on the compact axis of the slots that hold data
   const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
   const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
   const int prow = lane / CH, pch = lane % CH;  // this lane's row within a pass over the private tile, its physical chunk
-  // rows [cb, cb + 32) of a depth tensor -> the private tile (rows past the chunk's last column arrive as zeros)
+  WaveTileLoader<HD> own;
+  own.init(lane, a.D);
+  // columns [cb, cb + 32) of a depth tensor -> the private tile (rows past the chunk's last column arrive as zeros)
+  const bool partial = a.Lv != a.L;
   auto fetch = [&](const uint16_t* base, int64_t stride, int cb) {
-    const int nrows = min(32, c_end - cb);
-    const i32x4 rs = rsrc_words(base + (int64_t)cb * stride, (uint32_t)nrows * (uint32_t)stride * 2u);
-#pragma unroll
-    for (int i = 0; i < NPASS; i++) {
-      const int row = i * RPW + prow;
-      const int lch = pch ^ Tile<HD>::swz(row);  // chunks beyond the head dim: out of range, filled with zeros
-      lds_dma<16>(rs, lds_addr(wt + i * 512), lch * 8 < a.D ? row * (int)stride * 2 + lch * 16 : kPadOffset, 0);
-    }
+    if (partial)
+      own.fetch_mapped(wt, base, stride, cb, min(32, c_end - cb), (int64_t)a.T * a.L, a.L, a.Lv);
+    else
+      own.fetch(wt, base, stride, cb, min(32, c_end - cb));
   };
   auto landed = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
@@ -487,17 +513,29 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
 #pragma unroll
     for (int i = 0; i < NPASS; i++) {
       const int row = i * RPW + prow;
-      const i32x4 val = *reinterpret_cast<MODA_LDS const i32x4*>(wt + i * 512 + lane * 8);
+      i32x4 val = *reinterpret_cast<MODA_LDS const i32x4*>(wt + i * 512 + lane * 8);
       const int lch = pch ^ Tile<HD>::swz(row);
-      if (cb + row < c_end && lch * 8 < a.D)
-        *reinterpret_cast<i32x4*>(base + (int64_t)(cb + row) * stride + lch * 8) = val;
+      if (cb + row < c_end && lch * 8 < a.D) {
+        i32x4* dst = reinterpret_cast<i32x4*>(base + depth_row_of(a, cb + row) * stride + lch * 8);
+        if (a.accum_depth) {  // add to what the row holds (this lane is the only writer of its 16 bytes)
+          const i32x4 old = *dst;
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            float x0, x1, y0, y1;
+            unpack2<T>(val[w], x0, x1);
+            unpack2<T>(old[w], y0, y1);
+            val[w] = pack2<T>(x0 + y0, x1 + y1);
+          }
+        }
+        *dst = val;
+      }
     }
   };
 
-  for (int cb = t0 * a.L + wave * 32; cb < c_end; cb += 128) {
+  for (int cb = t0 * a.Lv + wave * 32; cb < c_end; cb += 128) {
     const int c = cb + n;
     // the column's visible rows: from its owner token's first row to the end of the chunk
-    const int qlo = c < c_end ? (c / a.L) * a.Gf : r_end;
+    const int qlo = c < c_end ? (c / a.Lv) * a.Gf : r_end;
     reads_done();
     fetch(kdp, a.skd.t, cb);
     landed();
@@ -688,6 +726,25 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   }
 }
 
+// Chunk-visible mode with a partially filled depth stream, not accumulating: the kernels above only visit the slots
+// that hold data, so the gradient rows of the other slots are written here (zeros).  One thread per 16 bytes of a
+// depth row; `rows`: depth rows per batch entry of the tensors (the whole packed axis for a packed batch).
+template <int HD>
+__global__ __launch_bounds__(256) void zero_unfilled_slots_kernel(const KArgs a, int64_t rows, int batches) {
+  constexpr int TPR = HD / 8;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int sub = (int)(gid % TPR);
+  int64_t rest = gid / TPR;
+  const int h = (int)(rest % a.Hkv);
+  rest /= a.Hkv;
+  const int64_t row = rest % rows;
+  const int64_t b = rest / rows;
+  if (b >= batches || 8 * sub >= a.D || (int)(row % a.L) < a.Lv) return;
+  const i32x4 z = {0, 0, 0, 0};
+  *reinterpret_cast<i32x4*>(a.dkd + b * a.sdkd.b + h * a.sdkd.h + row * a.sdkd.t + 8 * sub) = z;
+  *reinterpret_cast<i32x4*>(a.dvd + b * a.sdvd.b + h * a.sdvd.h + row * a.sdvd.t + 8 * sub) = z;
+}
+
 // Adds the fp32 partial sums of the row segments (in segment order: the result does not depend on which
 // workgroup finished first) and writes dk, dv in the tensor type.  One thread per 8 head-dim elements.
 template <typename T, int HD>
@@ -760,6 +817,17 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
       const hipError_t er = hipGetLastError();
       if (er != hipSuccess) return er;
     }
+  }
+  if (a.L > 0 && a.chunk && a.Lv != a.L && !a.accum_depth && (int64_t)a.B * a.T > 0) {
+    // packed batch: one row axis of all sequences (its length is the row-sum pitch / G), else B x T * L rows
+    const int64_t rows = a.cu ? (int64_t)(a.delta_pitch / a.Gf) * a.L : (int64_t)a.T * a.L;
+    const int batches = a.cu ? 1 : a.B;
+    const int64_t nthreads = rows * batches * a.Hkv * (HD / 8);
+    if ((nthreads + 255) / 256 >= (1ll << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((zero_unfilled_slots_kernel<HD>), dim3((unsigned)((nthreads + 255) / 256)), dim3(256), 0, stream, a,
+                       rows, batches);
+    const hipError_t ez = hipGetLastError();
+    if (ez != hipSuccess) return ez;
   }
   if constexpr (HD <= 128) if (depth_by_chunks && (int64_t)a.B * a.T > 0) {
     constexpr size_t csmem = (2 * 64 + 4 * 32) * HD * sizeof(uint16_t) + 2 * 64 * sizeof(float);

@@ -39,6 +39,13 @@ bool aligned(const void* p, const moda_hip_strides& s, int esize, bool vec16) {
 // below 16 MiB (tiles have at most 64 rows per pass).
 bool row_stride_ok(const moda_hip_strides& s, int esize) { return s.t >= 0 && s.t * esize < (1ll << 24); }
 
+// A partially filled depth stream is read through one descriptor per tile, anchored at the first column's token:
+// the byte offsets of a tile's 64 columns from that anchor -- up to 64 / Lv + 2 tokens of L rows -- must fit 31 bits.
+bool mapped_span_ok(const KArgs& a, const moda_hip_strides& s, int esize) {
+  if (a.L == 0 || a.Lv == a.L) return true;
+  return (int64_t)(64 / a.Lv + 2) * a.L * s.t * esize < (1ll << 31);
+}
+
 int value_dim(const moda_hip_desc* d) { return (int)(d->Dv > 0 ? d->Dv : d->D); }
 
 // The matrix-core kernels exist for tile widths 64, 128 and 256; any 16-bit head dim that is a multiple of 8 (whole
@@ -69,9 +76,7 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   if (d->mode == MODA_HIP_DEPTH_ONLY && d->L == 0) return MODA_HIP_EINVAL;
   if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L > 0 && d->chunk_tokens <= 0) return MODA_HIP_EINVAL;
   if (d->L_valid < 0 || d->L_valid > d->L) return MODA_HIP_EINVAL;
-  if (d->mode == MODA_HIP_CHUNK_VISIBLE && d->L_valid != 0 && d->L_valid != d->L) return MODA_HIP_EUNSUPPORTED;
   if (d->flags & ~(int32_t)MODA_HIP_FLAG_ACCUMULATE_DEPTH_GRADS) return MODA_HIP_EINVAL;
-  if ((d->flags & MODA_HIP_FLAG_ACCUMULATE_DEPTH_GRADS) && d->mode == MODA_HIP_CHUNK_VISIBLE) return MODA_HIP_EUNSUPPORTED;
   // 32-bit index space used for rows and flattened depth columns inside the kernels
   if (d->T * d->G >= (1ll << 30) || d->T * (d->L > 0 ? d->L : 1) >= (1ll << 30) || d->B * d->H * d->G >= (1ll << 20))
     return MODA_HIP_EUNSUPPORTED;
@@ -87,6 +92,7 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   a.hdiv = plain ? (int)d->G : 1;
   a.L = (int)d->L;
   a.Lv = d->L_valid > 0 ? (int)d->L_valid : (int)d->L;
+  if (a.Lv == 0) a.Lv = a.L = 0;
   a.Cb = d->mode == MODA_HIP_CHUNK_VISIBLE ? (int)(d->chunk_tokens > 0 ? d->chunk_tokens : 1) : 1;
   a.has_seq = d->mode != MODA_HIP_DEPTH_ONLY;
   a.causal = d->mode == MODA_HIP_CAUSAL || d->mode == MODA_HIP_CHUNK_VISIBLE || plain;
@@ -254,6 +260,7 @@ int moda_hip_fwd(const moda_hip_desc* d, const void* q, const void* k, const voi
     MODA_REQ_PTR(vd);
     MODA_REQ_ALIGN(kd, d->kd);
     MODA_REQ_ALIGN(vd, d->vd);
+    if (vec16 && !(mapped_span_ok(a, d->kd, es) && mapped_span_ok(a, d->vd, es))) return MODA_HIP_EUNSUPPORTED;
   }
   if ((rc = check_device(&a.compute_units))) return rc;
   a.q = (const uint16_t*)q;
@@ -362,6 +369,7 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
       MODA_REQ_ALIGN(vd, d->vd);
       MODA_REQ_ALIGN(dkd, d->dkd);
       MODA_REQ_ALIGN(dvd, d->dvd);
+      if (vec16 && !(mapped_span_ok(a, d->kd, es) && mapped_span_ok(a, d->vd, es))) return MODA_HIP_EUNSUPPORTED;
     }
     if (!workspace || workspace_bytes < delta_bytes_exact(a)) return MODA_HIP_EWORKSPACE;
     if ((uintptr_t)workspace % sizeof(float) != 0) return MODA_HIP_EALIGN;

@@ -29,7 +29,8 @@ namespace moda {
 using FwdLarge = RowLargePP;
 
 // ADDR bit 0: a (batch, head) slice is wider than 2 GiB (descriptors anchored per tile instead of 32-bit
-// offsets inside the slice); bit 1: packed variable-length batch; bit 2: no depth stream
+// offsets inside the slice); bit 1: packed variable-length batch; bit 2: no depth stream; bit 3: partially filled
+// depth stream (only Lv of a token's L slots hold data: depth tiles are loaded through the slot mapping)
 template <typename T, int HD, typename Shape, int ADDR>
 __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in) {
   constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST,
@@ -45,7 +46,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0;
   // bit 2: launched without a depth stream (the plain and sequence-only calls): the depth code is compiled out,
   // so that it cannot disturb the register allocation of their main loop
-  constexpr bool NODEPTH = (ADDR & 4) != 0;
+  constexpr bool NODEPTH = (ADDR & 4) != 0, PARTIAL = (ADDR & 8) != 0;
+  static_assert(!(NODEPTH && PARTIAL), "a partially filled depth stream is a depth stream");
   const int BH = a_in.B * a_in.Hq;
   const int bh = blockIdx.x % BH;
   int b = bh / a_in.Hq;
@@ -113,7 +115,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
       srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
-    if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
+    if (PARTIAL && it >= n_seq) {  // depth tile of a partially filled stream: rows through the slot mapping
+      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
+      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
+    } else if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
       const bool dep = !NODEPTH && it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
@@ -342,8 +347,16 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
       const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
       Own own;
       own.init(lane, a.D);
-      own.fetch(Kt, kdp, a.skd.t, c_beg, min(32, c_end - c_beg));
-      own.fetch(Vt, vdp, a.svd.t, c_beg, min(32, c_end - c_beg));
+      // rows [col0, col0 + 32) of the span (short at its end) into a private tile
+      auto fetch = [&](lds_ptr tile, const uint16_t* slice, int64_t stride, int col0) {
+        const int nrows = min(32, c_end - col0);
+        if (PARTIAL)
+          own.fetch_mapped(tile, slice, stride, col0, nrows, (int64_t)a.T * a.L, a.L, a.Lv);
+        else
+          own.fetch(tile, slice, stride, col0, nrows);
+      };
+      fetch(Kt, kdp, a.skd.t, c_beg);
+      fetch(Vt, vdp, a.svd.t, c_beg);
       const std::integral_constant<int, 1> one{};
       for (int j = 0; j < nh; j++) {
         const int col0 = c_beg + 32 * j;
@@ -351,7 +364,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         Own::template wait_but<Own::N>();  // K landed, V may still be on its way
         front(std::true_type{}, one, Kt, col0, dlo, dhi, []() {});
         Own::reads_done();
-        if (more) own.fetch(Kt, kdp, a.skd.t, col0 + 32, min(32, c_end - col0 - 32));
+        if (more) fetch(Kt, kdp, a.skd.t, col0 + 32);
         if (more)
           Own::template wait_but<Own::N>();  // V landed, the next K on its way
         else
@@ -361,7 +374,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         pv1.prefetch(oa, Vt);
         pv1.run(oa, Vt, P1, o);
         Own::reads_done();
-        if (more) own.fetch(Vt, vdp, a.svd.t, col0 + 32, min(32, c_end - col0 - 32));
+        if (more) fetch(Vt, vdp, a.svd.t, col0 + 32);
       }
     }
   }
@@ -398,7 +411,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
   lds_ptr smem = (lds_ptr)smem_raw;  // ring stage st: K tile at smem + st * 2*BN*HD, V tile right behind it
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, q4 = lane >> 4;
-  constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0;
+  constexpr bool WIDE = (ADDR & 1) != 0, VARLEN = (ADDR & 2) != 0, PARTIAL = (ADDR & 8) != 0;
   const int BH = a_in.B * a_in.Hq;
   const int bh = blockIdx.x % BH;
   int b = bh / a_in.Hq;
@@ -464,7 +477,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
       srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
-    if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
+    if (PARTIAL && it >= n_seq) {  // depth tile of a partially filled stream: rows through the slot mapping
+      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
+      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
+    } else if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
       const bool dep = it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
@@ -672,7 +688,7 @@ hipError_t launch_fwd_wide(const KArgs& a, hipStream_t stream) {
 
 template <typename T, int HD, int ADDR>
 hipError_t launch_fwd_t_addr(const KArgs& a, bool small, hipStream_t stream) {
-  if constexpr (HD > 128) return launch_fwd_wide<T, HD, ADDR & 3>(a, stream);
+  if constexpr (HD > 128) return launch_fwd_wide<T, HD, ADDR & 11>(a, stream);
   else {
     if (ADDR & 1) return launch_fwd_t_shape<T, HD, FwdLarge, ADDR>(a, stream);  // slices wider than 2 GiB: never a small launch
     if (small) return launch_fwd_t_shape<T, HD, RowSmall<HD>, ADDR>(a, stream);
@@ -687,7 +703,7 @@ hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
                                     std::max((int64_t)a.T * a.L * a.skd.t, (int64_t)a.T * a.L * a.svd.t));
   const bool wide = span > 0x7fffffffll;
   const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
-  switch ((wide ? 1 : 0) | (a.cu ? 2 : 0) | (a.L == 0 ? 4 : 0)) {
+  switch ((wide ? 1 : 0) | (a.cu ? 2 : 0) | (a.L == 0 ? 4 : 0) | (a.L > 0 && a.Lv != a.L ? 8 : 0)) {
     case 0: return launch_fwd_t_addr<T, HD, 0>(a, small, stream);
     case 1: return launch_fwd_t_addr<T, HD, 1>(a, small, stream);
     case 2: return launch_fwd_t_addr<T, HD, 2>(a, small, stream);
@@ -695,7 +711,11 @@ hipError_t launch_fwd_t(const KArgs& a, hipStream_t stream) {
     case 4: return launch_fwd_t_addr<T, HD, 4>(a, small, stream);
     case 5: return launch_fwd_t_addr<T, HD, 5>(a, small, stream);
     case 6: return launch_fwd_t_addr<T, HD, 6>(a, small, stream);
-    default: return launch_fwd_t_addr<T, HD, 7>(a, small, stream);
+    case 7: return launch_fwd_t_addr<T, HD, 7>(a, small, stream);
+    case 8: return launch_fwd_t_addr<T, HD, 8>(a, small, stream);
+    case 9: return launch_fwd_t_addr<T, HD, 9>(a, small, stream);
+    case 10: return launch_fwd_t_addr<T, HD, 10>(a, small, stream);
+    default: return launch_fwd_t_addr<T, HD, 11>(a, small, stream);
   }
 }
 

@@ -107,7 +107,8 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, cons
     const int64_t kb = g.b * ks.b + g.hkv * ks.h, vb = g.b * vs.b + g.hkv * vs.h;
     for (int c0 = lo; c0 < hi; c0 += 64) {
       const int col = c0 + lane;
-      const bool vis = col < hi;
+      // chunk-visible depth columns span several tokens: the slots without data among them are skipped
+      const bool vis = col < hi && !(phase == 1 && a.chunk && (col % a.L) >= a.Lv);
       float s = 0.f, dp = 0.f;
       if (vis) {
         for (int d = 0; d < D; d++) s += qs[wave][d] * ld<E>(kp, kb + (int64_t)col * ks.t + d);
@@ -141,7 +142,10 @@ __global__ __launch_bounds__(256) void generic_row_kernel(const KArgs a_in, cons
         const int d = lane + 64 * i;
         if (d < Dx) {
           float x = acc[i] * alpha;
-          for (int j = 0; j < nc; j++) x += pb[wave][j] * ld<E>(xp, xb + (int64_t)(c0 + j) * xs + d);
+          for (int j = 0; j < nc; j++) {
+            const float wj = pb[wave][j];  // the same in every lane; rows of weight zero (invisible columns) are not read
+            if (wj != 0.f) x += wj * ld<E>(xp, xb + (int64_t)(c0 + j) * xs + d);
+          }
           acc[i] = x;
         }
       }

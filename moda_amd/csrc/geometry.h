@@ -12,6 +12,15 @@ namespace moda {
 MODA_HD int imin(int a, int b) { return a < b ? a : b; }
 MODA_HD int imax(int a, int b) { return a > b ? a : b; }
 
+// Depth columns.  A depth tensor holds L slots per token (row t * L + l = slot l of token t) of which the first
+// Lv hold data.  The kernels count depth columns on the COMPACT axis of the slots that hold data: column
+// c = t * Lv + l; slots l >= Lv are never read.  With Lv == L (every slot filled) the compact axis is the row axis.
+MODA_HD int64_t depth_row_of(const KArgs& a, int c) {
+  if (a.Lv == a.L) return c;
+  const int t = c / a.Lv;
+  return (int64_t)t * a.L + (c - t * a.Lv);
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Query-row kernels (forward, dQ): a workgroup owns BM consecutive query rows of one (batch, query head)
 // and streams BN-column tiles: the sequence keys, then (when they go through the workgroup's ring) the
@@ -23,7 +32,7 @@ MODA_HD int imax(int a, int b) { return a > b ? a : b; }
 // together; a result >= the sequence's own tile count means the workgroup has nothing to do.
 MODA_HD int query_tile_of(int block, int BH, int BM, int Tq_grid) { return (Tq_grid + BM - 1) / BM - 1 - block / BH; }
 
-// Visible column intervals [0, shi) of the sequence keys and [dlo, dhi) of the flattened depth columns for
+// Visible column intervals [0, shi) of the sequence keys and [dlo, dhi) of the depth columns (compact axis) for
 // query row r (all zero for a row past the end).  Ld: depth slots per token, 0 when the launch has no depth stream.
 struct RowVis {
   int shi, dlo, dhi;
@@ -35,8 +44,8 @@ MODA_HD RowVis row_visibility(const KArgs& a, int r, int Ld) {
     if (a.has_seq) v.shi = a.causal ? t + 1 : a.T;
     if (Ld > 0) {
       const int lo_t = a.chunk ? (t / a.Cb) * a.Cb : t;
-      v.dlo = lo_t * a.L;
-      v.dhi = a.chunk ? (t + 1) * a.L : v.dlo + a.Lv;  // the token's filled slots
+      v.dlo = lo_t * a.Lv;
+      v.dhi = (t + 1) * a.Lv;
     }
   }
   return v;
@@ -64,8 +73,8 @@ MODA_HD RowTilePlan row_tile_plan(const KArgs& a, int qt, int BM, int BN, bool r
   }
   if (ring_depth) {
     const int lo_t = a.chunk ? (t_first / a.Cb) * a.Cb : t_first;
-    p.dep0 = lo_t * a.L;
-    p.n_dep = ((t_last + 1) * a.L - p.dep0 + BN - 1) / BN;
+    p.dep0 = lo_t * a.Lv;
+    p.n_dep = ((t_last + 1) * a.Lv - p.dep0 + BN - 1) / BN;
   }
   return p;
 }
@@ -74,15 +83,15 @@ MODA_HD int ring_tile_row0(const RowTilePlan& p, int it, int BN) {
   return it < p.n_seq ? it * BN : p.dep0 + (it - p.n_seq) * BN;
 }
 
-// Flattened depth columns [c_beg, c_end) that the `rows` query rows starting at rw0 (< Tq) can see.
+// Depth columns [c_beg, c_end) that the `rows` query rows starting at rw0 (< Tq) can see.
 struct DepthSpan {
   int c_beg, c_end;
 };
 MODA_HD DepthSpan own_depth_span(const KArgs& a, int rw0, int rows) {
   const int tw0 = rw0 / a.Gf, tw1 = (imin(a.Tq, rw0 + rows) - 1) / a.Gf;
   DepthSpan s;
-  s.c_beg = (a.chunk ? (tw0 / a.Cb) * a.Cb : tw0) * a.L;
-  s.c_end = (tw1 + 1) * a.L;
+  s.c_beg = (a.chunk ? (tw0 / a.Cb) * a.Cb : tw0) * a.Lv;
+  s.c_end = (tw1 + 1) * a.Lv;
   return s;
 }
 
@@ -97,7 +106,7 @@ MODA_HD void q_interval(const KArgs& a, bool dep, int col, int& lo, int& hi) {
     lo = a.causal ? col * a.Gf : 0;
     hi = a.Tq;
   } else {
-    const int w = col / a.L;
+    const int w = col / a.Lv;
     lo = w * a.Gf;
     hi = a.chunk ? imin(a.T, (w / a.Cb + 1) * a.Cb) * a.Gf : (w + 1) * a.Gf;
   }
@@ -120,7 +129,7 @@ MODA_HD ColTilePlan col_tile_plan(const KArgs& grid, const KArgs& a, int ct, int
   const int n_seq_tiles = grid.has_seq ? (grid.T + BN - 1) / BN : 0;
   p.active = true;
   p.dep = ct >= n_seq_tiles * nseg;
-  p.ncols = p.dep ? a.T * a.L : a.T;
+  p.ncols = p.dep ? a.T * a.Lv : a.T;
   p.seg = p.dep ? 0 : ct % nseg;
   int tile = p.dep ? ct - n_seq_tiles * nseg : ct / nseg;
   if (varlen && !p.dep && a.causal) {
@@ -160,7 +169,7 @@ inline int64_t row_kernel_blocks(const KArgs& a, int rows_per_block) {
 inline bool depth_by_chunks(const KArgs& a, int HD) { return HD <= 128 && a.L > 0 && a.chunk && (int64_t)a.Cb * a.Gf <= 64; }
 inline int64_t col_kernel_blocks(const KArgs& a, int HD, int BN, int nseg) {
   const int64_t n_seq_tiles = a.has_seq ? (a.T + BN - 1) / BN : 0;
-  const int64_t n_dep_tiles = (a.L > 0 && a.chunk && !depth_by_chunks(a, HD)) ? ((int64_t)a.T * a.L + BN - 1) / BN : 0;
+  const int64_t n_dep_tiles = (a.L > 0 && a.chunk && !depth_by_chunks(a, HD)) ? ((int64_t)a.T * a.Lv + BN - 1) / BN : 0;
   return (n_seq_tiles * nseg + n_dep_tiles) * a.B * a.Hkv;
 }
 inline int64_t delta_kernel_blocks(const KArgs& a, int rows_per_block) {

@@ -290,11 +290,19 @@ inline hipError_t allow_dynamic_lds(LdsAttrState& state, const void* kernel, siz
 // The compiler's hazard pass does not look inside inline assembly either: a vector-memory instruction
 // that reads a scalar register written by a vector-ALU instruction (v_readfirstlane, v_readlane of a
 // spilled scalar) fewer than five wait states earlier sees the register's OLD value.  The compiler places
-// such writes right in front of the block when scalar registers are short, so the block brings its own
-// wait states: s_mov (1) + s_nop 3 (4), which also covers the one wait state m0 needs.
-template <int BYTES>
+// such writes right in front of the block when scalar registers are short (the forward kernels: dozens of sites),
+// so the block brings its own wait states: s_mov (1) + s_nop 3 (4), which also covers the one wait state m0 needs.
+// A kernel whose compiled code is known to keep its distance (tests/test_inline_asm_hazards_cpu.py checks every
+// tile load of every kernel in the compiler's output) may ask for NOP = 0 -- through the loaders' last template
+// argument, or for a whole source file by defining MODA_DMA_NOP as 0 before including this header -- and save the
+// four cycles per load; m0 still gets its one wait state.
+#ifndef MODA_DMA_NOP
+#define MODA_DMA_NOP 3
+#endif
+template <int BYTES, int NOP = MODA_DMA_NOP>
 __device__ __forceinline__ void lds_dma(i32x4 rsrc, uint32_t lds_byte_addr, int voff, int soff) {
   static_assert(BYTES == 16 || BYTES == 4, "dwordx4 or dword");
+  static_assert(NOP == 0 || NOP == 3, "one wait state for m0, or five for scalars written by the vector ALU");
   // The scalar operands are wave-uniform by contract.  Under scalar-register pressure the compiler may
   // park such a value in a vector register and would then hand that register to the "s" operands
   // below; reading it back through readfirstlane (free when the value already sits in a scalar
@@ -306,13 +314,23 @@ __device__ __forceinline__ void lds_dma(i32x4 rsrc, uint32_t lds_byte_addr, int 
   rs[1] = __builtin_amdgcn_readfirstlane(rsrc[1]);
   rs[2] = __builtin_amdgcn_readfirstlane(rsrc[2]);
   rs[3] = __builtin_amdgcn_readfirstlane(rsrc[3]);
-  if (BYTES == 16)
+  if (BYTES == 16 && NOP == 3)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
                  : "memory", "m0");
-  else
+  else if (BYTES == 16)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
+                 : "memory", "m0");
+  else if (NOP == 3)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :
+                 : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
+                 : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
                  : "s"(m0v), "v"(voff), "s"(rs), "s"(so)
                  : "memory", "m0");
@@ -341,7 +359,21 @@ __device__ __forceinline__ uint32_t lds_addr(lds_cptr p) { return (uint32_t)(uin
 // zero-padded): past the end of every descriptor, so the range check fills the chunk with zeros.
 constexpr int kPadOffset = 0x7ffffff0;
 
-template <int HD, int ROWS, int NT>
+// Depth tiles when only Lv of a token's L slots hold data: the tile's columns are counted on the compact axis
+// (column c = token * Lv + slot, see geometry.h) and lie in rows token * L + slot of the tensor.  The loaders anchor
+// one descriptor at slot 0 of the first column's token; this is the row, relative to that anchor, of the tile's
+// row `rho`, given the first column's slot l0.
+__host__ __device__ __forceinline__ int mapped_row(int l0, int rho, int L, int Lv) {
+  const int l = l0 + rho, dw = l / Lv;
+  return dw * L + (l - dw * Lv);
+}
+// bytes the anchored descriptor covers: from the anchor row to the end of the slice (rows_total rows), capped
+__host__ __device__ __forceinline__ uint32_t mapped_bytes(int64_t anchor_row, int64_t rows_total, uint32_t stride_bytes) {
+  const int64_t left = (rows_total - anchor_row) * (int64_t)stride_bytes;
+  return left <= 0 ? 0u : left > 0x7fffffffll ? 0x7fffffffu : (uint32_t)left;
+}
+
+template <int HD, int ROWS, int NT, int NOP = MODA_DMA_NOP>
 struct AsyncTileLoader {
   static constexpr int CH = HD / 8;            // 16-byte chunks per row
   static constexpr int NW = NT / 64;           // waves
@@ -399,7 +431,7 @@ struct AsyncTileLoader {
   __device__ __forceinline__ void load_from(lds_ptr tile, const Source& s, int row0) const {
     const i32x4 rs = rsrc_words(s.base, s.nbytes);
 #pragma unroll
-    for (int i = 0; i < N; i++) lds_dma<16>(rs, lds_addr(tile + lds_elems(i)), s.voff, source_soffset(s, row0, i));
+    for (int i = 0; i < N; i++) lds_dma<16, NOP>(rs, lds_addr(tile + lds_elems(i)), s.voff, source_soffset(s, row0, i));
   }
   // bytes covered by the descriptor load() anchors at row `row0` of a slice that ends at row `row_end`
   __host__ __device__ __forceinline__ static uint32_t anchored_bytes(int64_t row_stride, int row0, int row_end) {
@@ -413,7 +445,22 @@ struct AsyncTileLoader {
     const i32x4 rs = rsrc_words(src + (int64_t)row0 * row_stride, anchored_bytes(row_stride, row0, row_end));
     const int voff = lane_offset((int)stride_bytes);
 #pragma unroll
-    for (int i = 0; i < N; i++) lds_dma<16>(rs, lds_addr(tile + lds_elems(i)), voff, rows_before(i) * (int)stride_bytes);
+    for (int i = 0; i < N; i++) lds_dma<16, NOP>(rs, lds_addr(tile + lds_elems(i)), voff, rows_before(i) * (int)stride_bytes);
+  }
+  // this lane's byte offset, relative to the anchor, in load i of a mapped depth tile (see mapped_row)
+  __host__ __device__ __forceinline__ int mapped_offset(int i, int l0, int L, int Lv, int stride_bytes) const {
+    return gchunk < 0 ? kPadOffset : mapped_row(l0, rows_before(i) + row_in_pass, L, Lv) * stride_bytes + gchunk * 16;
+  }
+  // compact depth columns [col0, col0 + ROWS) of a slice of rows_total rows with L slots per token, Lv of them filled
+  __device__ __forceinline__ void load_mapped(lds_ptr tile, const uint16_t* slice, int64_t row_stride, int col0,
+                                              int64_t rows_total, int L, int Lv) const {
+    const int w0 = __builtin_amdgcn_readfirstlane(col0 / Lv), l0 = col0 - w0 * Lv;
+    const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
+    const int64_t anchor = (int64_t)w0 * L;
+    const i32x4 rs = rsrc_words(slice + anchor * row_stride, mapped_bytes(anchor, rows_total, stride_bytes));
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      lds_dma<16, NOP>(rs, lds_addr(tile + lds_elems(i)), mapped_offset(i, l0, L, Lv, (int)stride_bytes), 0);
   }
   // s_waitcnt vmcnt(0): every outstanding vector-memory load of this wave has landed
   __device__ __forceinline__ static void wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -428,7 +475,7 @@ struct AsyncTileLoader {
 // A 32-row tile that ONE wave stages for itself (same swizzled layout, same zero fill past the end of the
 // source and past the tensors' head dim).  Nothing but the wave's own counters orders these loads: wait for
 // vmcnt before reading the tile, and for lgkmcnt(0) -- all LDS reads returned -- before loading over it.
-template <int HD>
+template <int HD, int NOP = MODA_DMA_NOP>
 struct WaveTileLoader {
   static constexpr int CH = HD / 8, RPW = 64 / CH, N = 32 / RPW;  // chunks per row, rows per load, loads per tile
   int prow, pch, d;
@@ -449,7 +496,24 @@ struct WaveTileLoader {
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const i32x4 rs = rsrc_words(base + row0 * row_stride, nrows > 0 ? (uint32_t)nrows * stride_bytes : 0u);
 #pragma unroll
-    for (int i = 0; i < N; i++) lds_dma<16>(rs, lds_addr(tile + i * 512), lane_offset(i, (int)stride_bytes), 0);
+    for (int i = 0; i < N; i++) lds_dma<16, NOP>(rs, lds_addr(tile + i * 512), lane_offset(i, (int)stride_bytes), 0);
+  }
+  // the same for a mapped depth tile (see mapped_row): offset relative to the anchor, rows >= nrows padded
+  __host__ __device__ __forceinline__ int mapped_offset(int i, int l0, int L, int Lv, int nrows, int stride_bytes) const {
+    const int row = i * RPW + prow;
+    const int lch = pch ^ Tile<HD>::swz(row);
+    return (lch * 8 < d && row < nrows) ? mapped_row(l0, row, L, Lv) * stride_bytes + lch * 16 : kPadOffset;
+  }
+  // compact depth columns [col0, col0 + nrows) of a slice of rows_total rows, L slots per token, Lv of them filled
+  __device__ __forceinline__ void fetch_mapped(lds_ptr tile, const uint16_t* slice, int64_t row_stride, int col0,
+                                               int nrows, int64_t rows_total, int L, int Lv) const {
+    const int w0 = __builtin_amdgcn_readfirstlane(col0 / Lv), l0 = col0 - w0 * Lv;
+    const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
+    const int64_t anchor = (int64_t)w0 * L;
+    const i32x4 rs = rsrc_words(slice + anchor * row_stride, nrows > 0 ? mapped_bytes(anchor, rows_total, stride_bytes) : 0u);
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      lds_dma<16, NOP>(rs, lds_addr(tile + i * 512), mapped_offset(i, l0, L, Lv, nrows, (int)stride_bytes), 0);
   }
   // at most K of this wave's vector-memory loads (the youngest) still in flight
   template <int K>

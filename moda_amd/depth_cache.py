@@ -94,15 +94,15 @@ class DepthCache:
     ``[B, T*L_max, H, D]`` buffers and the number of slots written so far, to be
     passed as ``cached_k, cached_v, depth_valid=n`` -- nothing is copied or rebuilt
     between layers (the reference re-stacks all previous layers for every layer,
-    vision_tasks/deit/models.py:383-387).  The buffers start as zeros because the
-    kernels read (and multiply by zero) the unwritten slots.  Inference/no-grad use
-    only: ``append`` writes in place."""
+    vision_tasks/deit/models.py:383-387).  The buffers are not initialised: the kernels
+    never read a slot that has not been written.  Inference/no-grad use only: ``append``
+    writes in place."""
 
     def __init__(self, B: int, T: int, L_max: int, H: int, D: int, dtype, device):
         self.shape = (B, T, H, D)
         self.L_max = L_max
-        self.k = torch.zeros(B, T * L_max, H, D, dtype=dtype, device=device)
-        self.v = torch.zeros(B, T * L_max, H, D, dtype=dtype, device=device)
+        self.k = torch.empty(B, T * L_max, H, D, dtype=dtype, device=device)
+        self.v = torch.empty(B, T * L_max, H, D, dtype=dtype, device=device)
         self.n = 0
 
     def append(self, k: torch.Tensor, v: torch.Tensor):

@@ -26,17 +26,18 @@ from torch import nn
 
 from . import _lib
 from .depth_cache import DepthCache, _reorg_bwd, _reorg_fwd, stack_depth
-from .ops import _raw_bwd, parallel_moda, parallel_moda_fwd
+from .ops import _chunk_tokens, _raw_bwd, _raw_fwd, parallel_moda, parallel_moda_chunk_visible
 
 
 class _TrainBuffers:
-    """Cache and gradient accumulators of one forward/backward pass, ``[B, T*L_max, H, D]`` each.  All four
-    start as zeros: the kernels read (and multiply by zero) slots that are not written yet."""
+    """Cache and gradient accumulators of one forward/backward pass, ``[B, T*L_max, H, D]`` each.  The
+    accumulators start as zeros; the cache needs no initialisation (the kernels never read a slot that has not
+    been written: ``depth_valid``)."""
 
     def __init__(self, B, T, L_max, H, D, dtype, device):
         self.shape, self.L_max = (B, T, H, D), L_max
-        self.k = torch.zeros(B, T * L_max, H, D, dtype=dtype, device=device)
-        self.v = torch.zeros_like(self.k)
+        self.k = torch.empty(B, T * L_max, H, D, dtype=dtype, device=device)
+        self.v = torch.empty_like(self.k)
         self.gk = torch.zeros_like(self.k)
         self.gv = torch.zeros_like(self.k)
 
@@ -49,12 +50,11 @@ class _StreamAttention(torch.autograd.Function):
 
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
-    def forward(ctx, q, k, v, token, buf, n, scale, G, is_causal):
-        o, lse = parallel_moda_fwd(q, k, v, None, scale, cached_k=buf.k if n else None,
-                                   cached_v=buf.v if n else None, moda_group_num=G, is_causal=is_causal,
-                                   depth_valid=n if n else None)
+    def forward(ctx, q, k, v, token, buf, n, scale, G, mode, chunk_tokens):
+        o, lse = _raw_fwd(mode, q, k, v, buf.k if n else None, buf.v if n else None, scale, G, chunk_tokens,
+                          depth_valid=n if n else None)
         ctx.save_for_backward(q, k, v, o, lse)
-        ctx.buf, ctx.n, ctx.scale, ctx.G, ctx.is_causal = buf, n, scale, G, is_causal
+        ctx.buf, ctx.n, ctx.scale, ctx.G, ctx.mode, ctx.chunk_tokens = buf, n, scale, G, mode, chunk_tokens
         ctx.set_materialize_grads(False)
         ctx.mark_non_differentiable(lse)
         return o, lse, token.new_zeros(())
@@ -65,15 +65,15 @@ class _StreamAttention(torch.autograd.Function):
         q, k, v, o, lse = ctx.saved_tensors
         buf, n = ctx.buf, ctx.n
         do = torch.zeros_like(o) if do is None else do.to(o.dtype)
-        mode = _lib.CAUSAL if ctx.is_causal else _lib.NONCAUSAL
+        mode, cb = ctx.mode, ctx.chunk_tokens
         dq, dk, dv = torch.empty_like(q), torch.empty(k.shape, dtype=k.dtype, device=k.device), \
             torch.empty(v.shape, dtype=v.dtype, device=v.device)
         if n:
-            _raw_bwd(mode, q, k, v, buf.k, buf.v, o, lse, do, ctx.scale, ctx.G, out=(dq, dk, dv, buf.gk, buf.gv),
+            _raw_bwd(mode, q, k, v, buf.k, buf.v, o, lse, do, ctx.scale, ctx.G, cb, out=(dq, dk, dv, buf.gk, buf.gv),
                      depth_valid=n, accumulate_depth=True)
         else:
-            _raw_bwd(mode, q, k, v, None, None, o, lse, do, ctx.scale, ctx.G, out=(dq, dk, dv, None, None))
-        return dq, dk, dv, None, None, None, None, None, None
+            _raw_bwd(mode, q, k, v, None, None, o, lse, do, ctx.scale, ctx.G, cb, out=(dq, dk, dv, None, None))
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
 class _StreamPush(torch.autograd.Function):
@@ -160,8 +160,12 @@ class DepthStream:
             "collected by the stream, not by autograd"
         return stack_depth([kv[0] for kv in self._layers]), stack_depth([kv[1] for kv in self._layers]), None
 
-    def attend(self, q, k, v, scale=None, moda_group_num=1, is_causal=True):
-        """``parallel_moda(q, k, v, cached_k, cached_v, ...)`` over what has been pushed so far."""
+    def attend(self, q, k, v, scale=None, moda_group_num=1, is_causal=True, chunk_rows=None):
+        """``parallel_moda(q, k, v, cached_k, cached_v, ...)`` over what has been pushed so far; with ``chunk_rows``
+        (query rows per chunk, the reference's 64) ``parallel_moda_chunk_visible`` instead: a token also sees the
+        depth slots of the earlier tokens of its chunk (causal by definition)."""
+        chunk_visible = chunk_rows is not None
+        assert not chunk_visible or is_causal, "chunk-visible attention is causal"
         if self._mode == "train" or (self._mode is None and self._inplace is not False and not self._used_context
                                      and torch.is_grad_enabled() and (q.requires_grad or k.requires_grad)):
             # the same argument contract as parallel_moda, which is bypassed here
@@ -174,8 +178,10 @@ class DepthStream:
             if self._token is None:
                 self._token = torch.zeros((), device=q.device)
             buf = self._train if self._n else None
+            mode = _lib.CHUNK_VISIBLE if chunk_visible else _lib.CAUSAL if is_causal else _lib.NONCAUSAL
+            cb = _chunk_tokens(moda_group_num, chunk_rows) if chunk_visible else 0
             o, _, self._token = _StreamAttention.apply(q, k, v, self._token, buf, self._n, scale, moda_group_num,
-                                                       is_causal)
+                                                       mode, cb)
             return o
         if self._n == 0:
             dk = dv = n = None
@@ -184,6 +190,10 @@ class DepthStream:
         else:
             dk, dv = stack_depth([kv[0] for kv in self._layers]), stack_depth([kv[1] for kv in self._layers])
             n = None
+        if chunk_visible:
+            return parallel_moda_chunk_visible(q=q, k=k, v=v, g=None, scale=scale, cu_seqlens=None, cached_k=dk,
+                                               cached_v=dv, moda_group_num=moda_group_num, head_first=False,
+                                               warn_shape=False, chunk_rows=chunk_rows, depth_valid=n)
         return parallel_moda(q=q, k=k, v=v, g=None, scale=scale, cu_seqlens=None, cached_k=dk, cached_v=dv,
                              moda_group_num=moda_group_num, is_causal=is_causal, head_first=False, warn_shape=False,
                              depth_valid=n)
@@ -202,8 +212,9 @@ class MoDAAttention(nn.Module):
     depth stream from their feed-forward layers."""
 
     def __init__(self, dim, num_heads=8, num_kv_heads=1, qkv_bias=False, attn_drop=0., proj_drop=0.,
-                 is_causal=False, ffn_kv=False):
+                 is_causal=False, ffn_kv=False, chunk_rows=None):
         super().__init__()
+        self.chunk_rows = chunk_rows  # not None: chunk-visible attention with chunks of that many query rows
         if dim % num_heads != 0:
             raise ValueError(f"dim ({dim}) must be divisible by num_heads ({num_heads})")
         if num_heads % num_kv_heads != 0:
@@ -237,7 +248,12 @@ class MoDAAttention(nn.Module):
         k, v = self._split_kv(self.kv(x))
         if stream is not None:
             assert depth_k is None and depth_v is None, "pass either a stream or explicit depth tensors"
-            o = stream.attend(q, k, v, scale=self.scale, moda_group_num=G, is_causal=self.is_causal)
+            o = stream.attend(q, k, v, scale=self.scale, moda_group_num=G, is_causal=self.is_causal,
+                              chunk_rows=self.chunk_rows)
+        elif self.chunk_rows is not None:
+            o = parallel_moda_chunk_visible(q=q, k=k, v=v, g=None, scale=self.scale, cu_seqlens=None, cached_k=depth_k,
+                                            cached_v=depth_v, moda_group_num=G, head_first=False, warn_shape=False,
+                                            chunk_rows=self.chunk_rows, depth_valid=depth_valid)
         else:
             o = parallel_moda(q=q, k=k, v=v, g=None, scale=self.scale, cu_seqlens=None, cached_k=depth_k,
                               cached_v=depth_v, moda_group_num=G, is_causal=self.is_causal, head_first=False,
@@ -255,7 +271,7 @@ class MoDAStack(nn.Module):
     block)."""
 
     def __init__(self, dim, depth, num_heads, num_kv_heads, mlp_ratio=4., qkv_bias=True, is_causal=False,
-                 post_norm=False, ffn_kv=False):
+                 post_norm=False, ffn_kv=False, chunk_rows=None):
         super().__init__()
         self.post_norm, self.ffn_kv = post_norm, ffn_kv
         self.blocks = nn.ModuleList()
@@ -263,7 +279,7 @@ class MoDAStack(nn.Module):
             blk = nn.Module()
             blk.norm1 = nn.LayerNorm(dim, eps=1e-6)
             blk.attn = MoDAAttention(dim, num_heads, num_kv_heads, qkv_bias=qkv_bias, is_causal=is_causal,
-                                     ffn_kv=ffn_kv)
+                                     ffn_kv=ffn_kv, chunk_rows=chunk_rows)
             blk.norm2 = nn.LayerNorm(dim, eps=1e-6)
             hidden = int(dim * mlp_ratio)
             blk.mlp = nn.Sequential(nn.Linear(dim, hidden), nn.GELU(), nn.Linear(hidden, dim))

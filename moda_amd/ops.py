@@ -468,10 +468,8 @@ def parallel_moda(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_
     ignored.  ``depth_valid`` (an extension): ``cached_k/v`` keep ``L`` slots per token
     but only the first ``depth_valid`` are visible -- the result equals that for the
     compacted ``[B, T*depth_valid, H, D]`` tensors, the gradients of the other slots are
-    zero, and a preallocated cache (``DepthCache``) need not be rebuilt per layer.  The kernels still
-    read the other slots and multiply them by zero: they must hold FINITE values (``DepthCache`` and
-    ``DepthStream`` start their buffers as zeros; a ``torch.empty`` buffer may hold NaN/Inf bit patterns
-    that would turn the outputs into NaN).
+    zero, and a preallocated cache (``DepthCache``) need not be rebuilt per layer.  The other slots are
+    never read: they may hold anything (an uninitialised ``torch.empty`` buffer included).
     """
     q, k, v, g, cached_k, cached_v, scale = _prepare_inputs(
         "parallel_moda", q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first, return_depth_grads,
@@ -498,27 +496,29 @@ def _chunk_tokens(moda_group_num: int, chunk_rows: Optional[int]) -> int:
 
 def parallel_moda_chunk_visible_fwd(q, k, v, g_cumsum, scale, cu_seqlens=None, cached_k=None, cached_v=None,
                                     moda_group_num=1, customized_BT=None, customized_BS=None, customized_BK=None,
-                                    customized_BV=None, customized_num_warps=None, chunk_rows=None):
+                                    customized_BV=None, customized_num_warps=None, chunk_rows=None, depth_valid=None):
     """moda_v16.py:498-633.  The tile-size knobs are accepted and ignored, ``customized_BT`` included (the
-    reference overwrites it with 64, moda_v16.py:581-585); ``chunk_rows`` sets the chunk size in query rows."""
+    reference overwrites it with 64, moda_v16.py:581-585); ``chunk_rows`` sets the chunk size in query rows,
+    ``depth_valid`` is that of ``parallel_moda``."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
     assert q.shape[2] == k.shape[2], "Implicit head-dimension GQA is not allowed."
     cb = _chunk_tokens(moda_group_num, chunk_rows)
     return _raw_fwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, scale, moda_group_num, cb,
-                    packed=_packed(cu_seqlens, q, moda_group_num))
+                    depth_valid=depth_valid, packed=_packed(cu_seqlens, q, moda_group_num))
 
 
 def parallel_moda_chunk_visible_bwd(q, k, v, o, g_cumsum, lse, do, scale=None, chunk_size=128, cu_seqlens=None,
                                     cached_k=None, cached_v=None, moda_group_num=1, customized_BT=None,
                                     customized_BS=None, customized_BK=None, customized_BV=None,
-                                    customized_num_warps=None, chunk_rows=None):
-    """moda_v16.py:2099-2343 (``customized_BT`` ignored as there, ``chunk_rows`` as in the forward)."""
+                                    customized_num_warps=None, chunk_rows=None, depth_valid=None):
+    """moda_v16.py:2099-2343 (``customized_BT`` ignored as there, ``chunk_rows``, ``depth_valid`` as in the forward)."""
     assert g_cumsum is None, "g_cumsum is not supported in this version"
     if scale is None:
         scale = q.shape[-1] ** -0.5
     cb = _chunk_tokens(moda_group_num, chunk_rows)
     dq, dk, dv, dkd, dvd = _raw_bwd(_lib.CHUNK_VISIBLE, q, k, v, cached_k, cached_v, o, lse, do, scale,
-                                    moda_group_num, cb, packed=_packed(cu_seqlens, q, moda_group_num))
+                                    moda_group_num, cb, depth_valid=depth_valid,
+                                    packed=_packed(cu_seqlens, q, moda_group_num))
     return dq, dk, dv, None, dkd, dvd
 
 
@@ -528,9 +528,9 @@ class ParallelMixtureOfDepthAttentionChunkVisibleFunction(torch.autograd.Functio
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, q, k, v, g, scale, cu_seqlens, cached_k=None, cached_v=None, moda_group_num=1,
-                chunk_rows=None):
+                chunk_rows=None, depth_valid=None):
         o, lse = _autograd_forward(ctx, parallel_moda_chunk_visible_fwd, q, k, v, g, scale, cu_seqlens, cached_k,
-                                   cached_v, moda_group_num, chunk_rows=chunk_rows)
+                                   cached_v, moda_group_num, chunk_rows=chunk_rows, depth_valid=depth_valid)
         ctx.mark_non_differentiable(lse)
         return o, lse
 
@@ -538,14 +538,15 @@ class ParallelMixtureOfDepthAttentionChunkVisibleFunction(torch.autograd.Functio
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, do, dlse_unused):
         dq, dk, dv, dkd, dvd = _autograd_backward(ctx, parallel_moda_chunk_visible_bwd, do)
-        return dq, dk, dv, None, None, None, dkd, dvd, None, None
+        return dq, dk, dv, None, None, None, dkd, dvd, None, None, None
 
 
 def parallel_moda_chunk_visible(q, k, v, g=None, cached_k=None, cached_v=None, scale=None, cu_seqlens=None,
                                 moda_group_num=1, head_first=False, need_lse=False, return_depth_grads=True,
                                 warn_shape=True, customized_BT=None, customized_BS=None, customized_BT_backward=None,
-                                customized_BS_backward=None, chunk_rows=None):
-    """Chunk-visible MoDA; signature of moda_v16.py:3614-3632 plus ``chunk_rows``.  A query of base
+                                customized_BS_backward=None, chunk_rows=None, depth_valid=None):
+    """Chunk-visible MoDA; signature of moda_v16.py:3614-3632 plus ``chunk_rows`` and ``depth_valid`` (the latter
+    as in ``parallel_moda``: only the first ``depth_valid`` slots of every token hold data).  A query of base
     token ``t`` additionally sees the depth slots of tokens ``floor(t/Cb)*Cb .. t`` with
     ``Cb = 64 // moda_group_num``.  The four ``customized_*`` arguments are accepted and dropped exactly as the
     reference's wrapper drops them (moda_v16.py:3646-3650: a chunk is 64 query rows whatever they say);
@@ -554,7 +555,7 @@ def parallel_moda_chunk_visible(q, k, v, g=None, cached_k=None, cached_v=None, s
         "parallel_moda_chunk_visible", q, k, v, g, cached_k, cached_v, scale, moda_group_num, head_first,
         return_depth_grads, warn_shape)
     o, lse = ParallelMixtureOfDepthAttentionChunkVisibleFunction.apply(
-        q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, chunk_rows)
+        q, k, v, g, scale, cu_seqlens, cached_k, cached_v, moda_group_num, chunk_rows, depth_valid)
     return (o, lse) if need_lse else o
 
 

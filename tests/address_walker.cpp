@@ -275,7 +275,19 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
         ctx(kname, (int)block, wave, lane, dep ? "ring depth tile" : "ring sequence tile");
         for (int i = 0; i < Loader::N; i++) {
           const uint32_t ldsK = kt + (uint32_t)ld.lds_elems(i) * 2, ldsV = ldsK + BN * HD * 2;
-          if (WIDE_ADDR) {
+          if (dep && a.Lv != a.L) {  // partially filled stream: one descriptor anchored at the first column's token
+            const int w0 = row0 / a.Lv, l0 = row0 - w0 * a.Lv;
+            const int64_t anchor = (int64_t)w0 * a.L, rows_total = (int64_t)a.T * a.L;
+            check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + anchor * a.skd.t,
+                      mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u),
+                      ld.mapped_offset(i, l0, a.L, a.Lv, (int)a.skd.t * 2), 0, 16, ldsK, lds_bytes, ld.gchunk < 0);
+            check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + anchor * a.svd.t,
+                      mapped_bytes(anchor, rows_total, (uint32_t)a.svd.t * 2u),
+                      ld.mapped_offset(i, l0, a.L, a.Lv, (int)a.svd.t * 2), 0, 16, ldsV, lds_bytes, ld.gchunk < 0);
+            // a lane in range must have fetched a slot that holds data
+            const int rel = mapped_row(l0, Loader::rows_before(i) + ld.row_in_pass, a.L, a.Lv);
+            if ((anchor + rel) % a.L >= a.Lv) fail("mapped depth tile reads slot %d of %d filled", (int)((anchor + rel) % a.L), a.Lv);
+          } else if (WIDE_ADDR) {
             const int row_end = dep ? a.T * a.L : a.T;
             const uint16_t* kb = dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h;
             const uint16_t* vb = dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h;
@@ -307,6 +319,19 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
             const int col0 = span.c_beg + 32 * j;
             const int nrows = imin(32, span.c_end - col0);
             for (int i = 0; i < Own::N; i++) {
+              if (a.Lv != a.L) {
+                const int w0 = col0 / a.Lv, l0 = col0 - w0 * a.Lv;
+                const int64_t anchor = (int64_t)w0 * a.L, rows_total = (int64_t)a.T * a.L;
+                const int vk = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.skd.t * 2);
+                const int vv = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.svd.t * 2);
+                check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + anchor * a.skd.t,
+                          nrows > 0 ? mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u) : 0u, vk, 0, 16, kt + i * 1024,
+                          lds_bytes, vk == kPadOffset);
+                check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + anchor * a.svd.t,
+                          nrows > 0 ? mapped_bytes(anchor, rows_total, (uint32_t)a.svd.t * 2u) : 0u, vv, 0, 16, vt + i * 1024,
+                          lds_bytes, vv == kPadOffset);
+                continue;
+              }
               const int voffk = own.lane_offset(i, (int)a.skd.t * 2), voffv = own.lane_offset(i, (int)a.svd.t * 2);
               check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + (int64_t)col0 * a.skd.t,
                         nrows > 0 ? (uint32_t)nrows * (uint32_t)a.skd.t * 2u : 0u, voffk, 0, 16, kt + i * 1024, lds_bytes,
@@ -378,14 +403,14 @@ void walk_dkv(const KArgs& a_in) {
       for (int nb = 0; nb < NB; nb++) {
         const int c = plan.c_first + kblk * (16 * NB) + 16 * nb + n;
         const bool valid = c < plan.ncols;
-        const bool live = valid && !(dep && (c % a.L) >= a.Lv);
+        const int64_t crow = dep ? depth_row_of(a, c) : c;
         ctx("dkv_kernel", (int)block, wave, lane, "stationary K / V rows");
         const uint16_t* src = role_b ? (dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h)
                                      : (dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h);
         const int64_t st = role_b ? (dep ? a.svd.t : a.sv.t) : (dep ? a.skd.t : a.sk.t);
         const char* sname = role_b ? (dep ? "vd" : "v") : (dep ? "kd" : "k");
         for (int ks = 0; ks < KS; ks++)
-          if (live && 32 * ks + 8 * q4 < a.D) check_access(sname, src + (int64_t)c * st + 32 * ks + 8 * q4, 16, false);
+          if (valid && 32 * ks + 8 * q4 < a.D) check_access(sname, src + crow * st + 32 * ks + 8 * q4, 16, false);
         if (!valid) continue;
         ctx("dkv_kernel", (int)block, wave, lane, "gradient rows");
         if (nseg > 1 && !dep) {  // a row segment: fp32 partial sums, all HD columns of the tile width
@@ -396,10 +421,10 @@ void walk_dkv(const KArgs& a_in) {
           continue;
         }
         const char* oname = role_b ? (dep ? "dkd" : "dk") : (dep ? "dvd" : "dv");
-        uint16_t* outp = !role_b ? (dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)c * a.sdvd.t
-                                        : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t)
-                                 : (dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)c * a.sdkd.t
-                                        : a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t);
+        uint16_t* outp = !role_b ? (dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + crow * a.sdvd.t
+                                        : a.dv + b * a.sdv.b + hkv * a.sdv.h + crow * a.sdv.t)
+                                 : (dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + crow * a.sdkd.t
+                                        : a.dk + b * a.sdk.b + hkv * a.sdk.h + crow * a.sdk.t);
         for (int d = 0; d < MB; d++)
           if (16 * d + 4 * q4 < a.D) check_access(oname, outp + 16 * d + 4 * q4, 8, true);
       }
@@ -479,7 +504,7 @@ void walk_chunk_depth(const KArgs& a_in) {
     const KArgs a = seq_args(a_in, b);
     const int t0 = chunk * a.Cb;
     if (t0 >= a.T) continue;
-    const int t1 = imin(a.T, t0 + a.Cb), r0 = t0 * a.Gf, r_end = t1 * a.Gf, c_end = t1 * a.L;
+    const int t1 = imin(a.T, t0 + a.Cb), r0 = t0 * a.Gf, r_end = t1 * a.Gf, c_end = t1 * a.Lv;
     if (r_end - r0 > BM) fail("chunk_depth_kernel: a chunk of %d query rows", r_end - r0);
     for (int tid = 0; tid < 256; tid++) {
       const int lane = tid & 63, wave = tid >> 6;
@@ -500,24 +525,59 @@ void walk_chunk_depth(const KArgs& a_in) {
       }
       const int prow = lane / CH, pch = lane % CH;
       const uint32_t wt = (uint32_t)(2 * BM * HD + wave * 32 * HD) * 2;
-      for (int cb = t0 * a.L + wave * 32; cb < c_end; cb += 128) {
+      WaveTileLoader<HD> own;
+      own.init(lane, a.D);
+      for (int cb = t0 * a.Lv + wave * 32; cb < c_end; cb += 128) {
         const int nrows = imin(32, c_end - cb);
         for (int i = 0; i < NPASS; i++) {
           const int row = i * RPW + prow, lch = pch ^ Tile<HD>::swz(row);
           const bool pad = !(lch * 8 < a.D);
           ctx("chunk_depth_kernel", (int)block, wave, lane, "depth K / V rows");
-          check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + (int64_t)cb * a.skd.t, (uint32_t)nrows * (uint32_t)a.skd.t * 2u,
-                    pad ? kPadOffset : row * (int)a.skd.t * 2 + lch * 16, 0, 16, wt + i * 1024, lds_bytes, pad);
-          check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + (int64_t)cb * a.svd.t, (uint32_t)nrows * (uint32_t)a.svd.t * 2u,
-                    pad ? kPadOffset : row * (int)a.svd.t * 2 + lch * 16, 0, 16, wt + i * 1024, lds_bytes, pad);
+          if (a.Lv != a.L) {
+            const int w0 = cb / a.Lv, l0 = cb - w0 * a.Lv;
+            const int64_t anchor = (int64_t)w0 * a.L, rows_total = (int64_t)a.T * a.L;
+            const int vk = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.skd.t * 2);
+            const int vv = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.svd.t * 2);
+            check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + anchor * a.skd.t,
+                      mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u), vk, 0, 16, wt + i * 1024, lds_bytes, vk == kPadOffset);
+            check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + anchor * a.svd.t,
+                      mapped_bytes(anchor, rows_total, (uint32_t)a.svd.t * 2u), vv, 0, 16, wt + i * 1024, lds_bytes, vv == kPadOffset);
+          } else {
+            const int vk = own.lane_offset(i, (int)a.skd.t * 2), vv = own.lane_offset(i, (int)a.svd.t * 2);
+            check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + (int64_t)cb * a.skd.t, (uint32_t)nrows * (uint32_t)a.skd.t * 2u,
+                      vk, 0, 16, wt + i * 1024, lds_bytes, pad);
+            check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + (int64_t)cb * a.svd.t, (uint32_t)nrows * (uint32_t)a.svd.t * 2u,
+                      vv, 0, 16, wt + i * 1024, lds_bytes, pad);
+          }
           ctx("chunk_depth_kernel", (int)block, wave, lane, "depth gradient rows");
           if (cb + row < c_end && !pad) {
-            check_access("dkd", a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)(cb + row) * a.sdkd.t + lch * 8, 16, true);
-            check_access("dvd", a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)(cb + row) * a.sdvd.t + lch * 8, 16, true);
+            const int64_t prow_t = depth_row_of(a, cb + row);
+            check_access("dkd", a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + prow_t * a.sdkd.t + lch * 8, 16, true);
+            check_access("dvd", a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + prow_t * a.sdvd.t + lch * 8, 16, true);
           }
         }
       }
     }
+  }
+}
+
+// the gradient rows of the slots without data (chunk-visible mode with a partially filled stream)
+template <int HD>
+void walk_zero_unfilled(const KArgs& a) {
+  constexpr int TPR = HD / 8;
+  const int64_t rows = a.cu ? (int64_t)(a.delta_pitch / a.Gf) * a.L : (int64_t)a.T * a.L;
+  const int batches = a.cu ? 1 : a.B;
+  const int64_t nthreads = rows * batches * a.Hkv * TPR;
+  for (int64_t gid = 0; gid < (nthreads + 255) / 256 * 256; gid++) {
+    const int sub = (int)(gid % TPR);
+    int64_t rest = gid / TPR;
+    const int h = (int)(rest % a.Hkv);
+    rest /= a.Hkv;
+    const int64_t row = rest % rows, b = rest / rows;
+    if (b >= batches || 8 * sub >= a.D || (int)(row % a.L) < a.Lv) continue;
+    ctx("zero_unfilled_slots_kernel", (int)(gid / 256), (int)(gid % 256) >> 6, (int)(gid & 63), "gradient rows of empty slots");
+    check_access("dkd", a.dkd + b * a.sdkd.b + h * a.sdkd.h + row * a.sdkd.t + 8 * sub, 16, true);
+    check_access("dvd", a.dvd + b * a.sdvd.b + h * a.sdvd.h + row * a.sdvd.t + 8 * sub, 16, true);
   }
 }
 
@@ -628,6 +688,7 @@ void walk_all(const Case& c, const KArgs& a) {
     require_full("dv");
   }
   if (a.L > 0) {
+    if (a.chunk && a.Lv != a.L) walk_zero_unfilled<HD>(a);
     if (a.chunk) {
       if constexpr (HD <= 128) {
         if (depth_by_chunks(a, HD)) walk_chunk_depth<HD>(a);

@@ -79,7 +79,13 @@ FIXED = [
     (1, 333, 2, 128, 0, 4, "plain", 0, 0),
     (1, 200, 2, 120, 3, 4, "causal", 0, 0),
     (1, 90, 1, 8, 2, 2, "causal", 0, 0),
-    (2, 64, 2, 64, 4, 2, "causal", 0, 2),          # partially filled depth stream
+    (2, 64, 2, 64, 4, 2, "causal", 0, 2),          # partially filled depth stream: tile loads through the slot mapping
+    (1, 150, 2, 128, 7, 4, "noncausal", 0, 3),
+    (2, 100, 1, 64, 5, 1, "depth_only", 0, 1),
+    (1, 300, 2, 128, 6, 4, "chunk_visible", 16, 4),  # ... chunks within one query tile (chunk kernel)
+    (1, 260, 1, 64, 3, 4, "chunk_visible", 40, 2),   # ... and above it (ring depth tiles, depth column tiles)
+    (1, 200, 2, 192, 5, 2, "chunk_visible", 16, 3),  # ... on the 256-wide tiles
+    (2, 130, 2, 256, 12, 1, "causal", 0, 5),
     (2, 130, 2, 192, 6, 4, "chunk_visible", 16, 0),
     (1, 700, 1, 256, 3, 2, "chunk_visible", 64, 0),
     (1, 197, 3, 160, 12, 1, "noncausal", 0, 0),

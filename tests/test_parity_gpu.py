@@ -604,39 +604,58 @@ def test_slices_wider_than_32bit_offsets(gpu_device):
 
 
 @pytest.mark.parametrize("case", [
-    # (B, T, H, D, L, valid, G, mode, dtype)
-    (2, 150, 2, 64, 5, 3, 2, "causal", torch.bfloat16),
-    (1, 333, 2, 128, 6, 1, 4, "causal", torch.bfloat16),
-    (2, 197, 3, 64, 12, 7, 1, "noncausal", torch.float16),
-    (2, 97, 2, 128, 4, 4, 1, "causal", torch.bfloat16),
-    (2, 130, 2, 64, 9, 2, 2, "depth_only", torch.bfloat16),
-    (1, 70, 2, 96, 5, 2, 2, "causal", torch.bfloat16),   # generic kernels (head dim 96)
-    (1, 60, 2, 64, 3, 2, 1, "causal", torch.float32),    # generic kernels (fp32)
+    # (B, T, H, D, L, valid, G, mode, dtype, chunk tokens)
+    (2, 150, 2, 64, 5, 3, 2, "causal", torch.bfloat16, 0),
+    (1, 333, 2, 128, 6, 1, 4, "causal", torch.bfloat16, 0),
+    (2, 197, 3, 64, 12, 7, 1, "noncausal", torch.float16, 0),
+    (2, 97, 2, 128, 4, 4, 1, "causal", torch.bfloat16, 0),
+    (2, 130, 2, 64, 9, 2, 2, "depth_only", torch.bfloat16, 0),
+    (1, 70, 2, 96, 5, 2, 2, "causal", torch.bfloat16, 0),    # head dim zero-padded to 128
+    (1, 70, 2, 36, 5, 2, 2, "causal", torch.bfloat16, 0),    # vector-ALU kernels (head dim not a multiple of 8)
+    (1, 60, 2, 64, 3, 2, 1, "causal", torch.float32, 0),     # vector-ALU kernels (fp32)
+    (1, 300, 2, 256, 5, 2, 2, "causal", torch.bfloat16, 0),  # 256-wide tiles: depth columns through the ring
+    (3, 2100, 1, 128, 3, 2, 2, "causal", torch.bfloat16, 0),  # the throughput launch shape
+    # chunk-visible: chunks within one query tile (the waves' own depth tiles, the chunk kernel), above it (ring
+    # depth tiles, depth column tiles), on the 256-wide tiles, on the vector-ALU kernels
+    (1, 300, 2, 128, 6, 4, 4, "chunk_visible", torch.bfloat16, 16),
+    (2, 130, 1, 64, 7, 1, 2, "chunk_visible", torch.float16, 8),
+    (1, 260, 1, 64, 3, 2, 4, "chunk_visible", torch.bfloat16, 40),
+    (1, 400, 2, 128, 5, 3, 4, "chunk_visible", torch.bfloat16, 32),
+    (1, 200, 2, 192, 5, 3, 2, "chunk_visible", torch.float16, 16),
+    (1, 90, 2, 32, 4, 3, 2, "chunk_visible", torch.float32, 8),
 ])
 def test_partially_filled_depth_stream(gpu_device, case):
     """depth_valid = v on the L-slot tensors == the compacted [B, T*v, H, D] tensors (the oracle's
-    definition); the unused slots hold large finite junk and must get exactly zero gradient."""
+    definition).  The unused slots hold NaN, Inf and huge finite values -- an uninitialised cache -- which
+    must neither reach any output nor be read; their gradients must come out exactly zero."""
     from moda_amd import ops
 
-    B, T, H, D, L, valid, G, mode, dtype = case
+    B, T, H, D, L, valid, G, mode, dtype, cb = case
     say(f"CASE partial-depth {case}")
     inp = oracle.make_inputs(B, T, H, D, L, G, seed=29, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
     junk = torch.Generator().manual_seed(5)
     for n in ("kd", "vd"):
         x = inp[n].reshape(B, T, L, H, D)
-        x[:, :, valid:] = (30.0 * torch.randn(x[:, :, valid:].shape, generator=junk)).to(dtype)
+        fill = 30.0 * torch.randn(x[:, :, valid:].shape, generator=junk)
+        pick = torch.rand(fill.shape, generator=junk)
+        fill[pick < 0.3] = float("nan")
+        fill[(pick >= 0.3) & (pick < 0.45)] = float("inf")
+        fill[(pick >= 0.45) & (pick < 0.6)] = float("-inf")
+        x[:, :, valid:] = fill.to(dtype)
     comp = dict(inp)
     comp["kd"] = oracle.compact_depth(inp["kd"], T, valid).contiguous()
     comp["vd"] = oracle.compact_depth(inp["vd"], T, valid).contiguous()
     scale = D ** -0.5
-    ref = oracle.moda_dense_fwd_bwd(comp, scale, G, mode, 0)
+    ref = oracle.moda_dense_fwd_bwd(comp, scale, G, mode, cb)
     ref["dkd"] = oracle.scatter_depth_grad(ref["dkd"], T, L)
     ref["dvd"] = oracle.scatter_depth_grad(ref["dvd"], T, L)
     dev = to_dev(inp, gpu_device)
     m = MODE_ID[mode]
-    o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], scale, G, 0, depth_valid=valid)
+    o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], scale, G, cb, depth_valid=valid)
+    # the gradient buffers start as NaN: every element must be written
+    out = tuple(None if dev[n] is None else torch.full_like(dev[n], float("nan")) for n in ("q", "k", "v", "kd", "vd"))
     dq, dk, dv, dkd, dvd = ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], o, lse, dev["do"], scale,
-                                        G, 0, depth_valid=valid)
+                                        G, cb, depth_valid=valid, out=out)
     got = {"o": o, "lse": lse, "dq": dq, "dk": dk, "dv": dv, "dkd": dkd, "dvd": dvd}
     compare_all(got, ref, dtype, f"partial-depth {case}")
     for n in ("dkd", "dvd"):
@@ -677,6 +696,11 @@ def test_depth_cache_append_in_place(gpu_device):
     (1, 50, 2, 96, 3, 2, "causal", torch.bfloat16),     # matrix kernels, head dim zero-padded to 128
     (1, 50, 2, 36, 3, 2, "causal", torch.bfloat16),     # vector-ALU kernels (head dim not a multiple of 8)
     (2, 40, 1, 32, 4, 2, "noncausal", torch.float32),   # vector-ALU kernels (fp32)
+    # chunk-visible: the chunk kernel, depth column tiles (narrow and 256-wide tiles), vector-ALU kernels
+    (1, 150, 2, 128, 4, 4, "chunk_visible:16", torch.bfloat16),
+    (1, 200, 1, 64, 3, 4, "chunk_visible:40", torch.float16),
+    (1, 130, 2, 160, 3, 2, "chunk_visible:16", torch.bfloat16),
+    (1, 60, 1, 32, 3, 2, "chunk_visible:8", torch.float32),
 ])
 def test_depth_gradients_accumulate_over_layers(gpu_device, case):
     """The accumulate flag of the backward: the attention that saw n slots ADDS its depth gradients to slots
@@ -688,6 +712,9 @@ def test_depth_gradients_accumulate_over_layers(gpu_device, case):
 
     B, T, H, D, L, G, mode, dtype = case
     say(f"CASE accumulate-depth-grads {case}")
+    cb = 0
+    if ":" in mode:
+        mode, cb = mode.split(":")[0], int(mode.split(":")[1])
     m = MODE_ID[mode]
     scale = D ** -0.5
     base = oracle.make_inputs(B, T, H, D, L, G, seed=61, dtype=dtype, std=0.5, depth_only=(mode == "depth_only"))
@@ -702,15 +729,15 @@ def test_depth_gradients_accumulate_over_layers(gpu_device, case):
         comp = dict(layer)
         comp["kd"] = oracle.compact_depth(kd, T, n).contiguous()
         comp["vd"] = oracle.compact_depth(vd, T, n).contiguous()
-        ref = oracle.moda_dense_fwd_bwd(comp, scale, G, mode, 0)
+        ref = oracle.moda_dense_fwd_bwd(comp, scale, G, mode, cb)
         ref_k += oracle.scatter_depth_grad(ref["dkd"], T, L).float()
         ref_v += oracle.scatter_depth_grad(ref["dvd"], T, L).float()
         dev = to_dev(layer, gpu_device)
-        o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], kd_dev, vd_dev, scale, G, 0, depth_valid=n)
+        o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], kd_dev, vd_dev, scale, G, cb, depth_valid=n)
         dq = torch.empty_like(dev["q"])
         dk = None if dev["k"] is None else torch.empty_like(dev["k"])
         dv = None if dev["v"] is None else torch.empty_like(dev["v"])
-        ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], kd_dev, vd_dev, o, lse, dev["do"], scale, G, 0,
+        ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], kd_dev, vd_dev, o, lse, dev["do"], scale, G, cb,
                      out=(dq, dk, dv, acc_k, acc_v), depth_valid=n, accumulate_depth=True)
         check("dq", dq, ref["dq"], dtype, f"layer {n}")
     # L additions, each rounded to the tensor type: the tolerance of one rounding per addition
@@ -1005,10 +1032,21 @@ def _oracle_parallel_moda(q, k, v, g=None, scale=None, cu_seqlens=None, cached_k
     return o.to(q.dtype)
 
 
+def _oracle_parallel_moda_chunk_visible(q, k, v, g=None, scale=None, cu_seqlens=None, cached_k=None, cached_v=None,
+                                        moda_group_num=1, head_first=False, warn_shape=True, chunk_rows=None,
+                                        depth_valid=None):
+    assert depth_valid is None
+    o, _ = oracle.moda_dense(q, k, v, cached_k, cached_v, scale, moda_group_num, "chunk_visible",
+                             (chunk_rows or 64) // moda_group_num)
+    return o.to(q.dtype)
+
+
 @pytest.mark.parametrize("variant", [
-    # (causal, post_norm, ffn_kv)
-    (False, False, False), (True, False, False), (False, True, False), (True, False, True), (False, True, True),
-], ids=lambda v: f"{'causal' if v[0] else 'noncausal'}{'-postnorm' if v[1] else ''}{'-ffnkv' if v[2] else ''}")
+    # (causal, post_norm, ffn_kv, chunk rows or None)
+    (False, False, False, None), (True, False, False, None), (False, True, False, None), (True, False, True, None),
+    (False, True, True, None), (True, False, False, 32), (True, True, True, 64),
+], ids=lambda v: f"{'causal' if v[0] else 'noncausal'}{'-postnorm' if v[1] else ''}{'-ffnkv' if v[2] else ''}"
+                 f"{'-chunk%d' % v[3] if v[3] else ''}")
 def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, variant):
     """A three-block stack (layer norm, MoDAAttention, MLP, one DepthStream; pre- or post-norm, optionally
     with K/V of the block output pushed as well) trained one step on the HIP operator with the in-place depth
@@ -1018,11 +1056,11 @@ def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, variant):
     import moda_amd
     from moda_amd import depth_cache, modules
 
-    causal, post_norm, ffn_kv = variant
+    causal, post_norm, ffn_kv, chunk_rows = variant
     torch.manual_seed(41)
     dim, depth, heads, kv_heads, B, N = 256, 3, 4, 2, 2, 70
     model = moda_amd.MoDAStack(dim, depth, heads, kv_heads, is_causal=causal, post_norm=post_norm,
-                               ffn_kv=ffn_kv).to(gpu_device).to(torch.bfloat16)
+                               ffn_kv=ffn_kv, chunk_rows=chunk_rows).to(gpu_device).to(torch.bfloat16)
     x = (0.5 * torch.randn(B, N, dim, device=gpu_device)).to(torch.bfloat16)
     w = torch.randn(B, N, dim, device=gpu_device).to(torch.bfloat16)
 
@@ -1051,6 +1089,7 @@ def test_attention_stack_with_depth_stream(gpu_device, monkeypatch, variant):
     with torch.no_grad():
         y_inplace = model(x).float()
     monkeypatch.setattr(modules, "parallel_moda", _oracle_parallel_moda)
+    monkeypatch.setattr(modules, "parallel_moda_chunk_visible", _oracle_parallel_moda_chunk_visible)
     monkeypatch.setattr(modules, "stack_depth", lambda layers: oracle.depth_cache_ref(list(layers)))
     y_ref, dx_ref, g_ref = step(inplace=False)
 
