@@ -5,7 +5,7 @@
  *
  * Every pointer that names tensor data is a DEVICE pointer.  Strides are in
  * elements; the innermost (head-dim) stride is always 1.  For the matrix-core
- * kernels (bf16/fp16, head dim a multiple of 8 up to 256, Dv == D) every row must be 16-byte
+ * kernels (bf16/fp16, head dims D and Dv multiples of 8 up to 256) every row must be 16-byte
  * aligned (base pointer and all strides multiples of 8 elements) and a row
  * stride must stay below 16 MiB; every other combination runs on vector-ALU
  * kernels that need element alignment only.  All work is enqueued on the hipStream_t passed
@@ -123,7 +123,8 @@ typedef struct moda_hip_desc {
   moda_hip_strides q, k, v, kd, vd, o, d_o, dq, dk, dv, dkd, dvd;
   const int32_t* cu_seqlens; /* packed variable-length batch (see above): DEVICE array of B + 1 offsets, else NULL */
   int64_t total_tokens;      /* with cu_seqlens: cu_seqlens[B], the length of the packed token axis              */
-  int64_t Dv;                /* head dim of v, vd, o, do, dv, dvd; 0 = D.  Dv != D runs on the vector-ALU kernels */
+  int64_t Dv;                /* head dim of v, vd, o, do, dv, dvd; 0 = D (the reference takes any K, V <= 256,
+                                moda_v14.py:423-437) */
   const int32_t* cu_seqlens_host; /* optional HOST copy of the B + 1 offsets of cu_seqlens (checked against T and
                                      total_tokens), else NULL; see "Packed variable-length batch" above */
 } moda_hip_desc;

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         i32x4 z = {0, 0, 0, 0};
-        Sr[nb][ks] = (valid[nb] && 32 * ks + 8 * q4 < a.D)
+        Sr[nb][ks] = (valid[nb] && 32 * ks + 8 * q4 < (role_b ? a.Dv : a.D))
                          ? *reinterpret_cast<const i32x4*>(src + crow * st + 32 * ks + 8 * q4)
                          : z;
       }
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
 
   using Loader = AsyncTileLoader<HD, BM, 512>;
   Loader ld;
-  ld.init(tid, a.D);
+  ld.init(tid);
   // Producer.  The global -> LDS loads of one tile are NOT issued back to back: forty wave-wide
   // loads arriving at once queue up in the CU's address unit and every wave would sit on its issue
   // for hundreds of cycles.  prep() fixes the descriptors of the next tile (wave-uniform, scalar
@@ -130,8 +130,8 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
   // wave's statistic) that step down one tile per call: the scalar unit then has a few adds per trip
   // instead of a dozen dependent 64-bit multiplies.
   const uint32_t q_row_bytes = (uint32_t)a.sq.t * 2u, do_row_bytes = (uint32_t)a.sdo.t * 2u;
-  const int voff_q = ld.lane_offset((int)q_row_bytes);
-  const int voff_do = ld.lane_offset((int)do_row_bytes);
+  const int voff_q = ld.lane_offset((int)q_row_bytes, a.D);
+  const int voff_do = ld.lane_offset((int)do_row_bytes, a.Dv);
   // wave 0 fetches lse ([B, Tq, Hq]: one dword every Hq), wave 1 delta ([B, Hq, Tq]: contiguous)
   const int voff_stat = wave == 0 ? lane * a.Hq * 4 : lane * 4;
   const uint32_t stat_row_bytes = wave == 0 ? (uint32_t)a.Hq * 4u : 4u;
@@ -385,6 +385,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
       uint16_t* outp;
       float mul;
       const int64_t crow = column_row(nb);
+      const int width = role_b ? a.D : a.Dv;  // head dim of the gradient this role writes
       if (!role_b) {  // dV
         outp = dep ? a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + crow * a.sdvd.t
                    : a.dv + b * a.sdv.b + hkv * a.sdv.h + crow * a.sdv.t;
@@ -399,7 +400,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
         // old values of all pieces fetched up front the kernel would not fit its registers
 #pragma unroll
         for (int d = 0; d < MB; d++) {
-          if (16 * d + 4 * q4 < a.D) {
+          if (16 * d + 4 * q4 < width) {
             i32x2* dst = reinterpret_cast<i32x2*>(outp + 16 * d + 4 * q4);
             const i32x2 old = *dst;
             float o0, o1, o2, o3;
@@ -418,7 +419,7 @@ __global__ __launch_bounds__(512) void dkv_kernel(const KArgs a_in) {
           i32x2 w;
           w[0] = pack2<T>(acc[d][nb][0] * mul, acc[d][nb][1] * mul);
           w[1] = pack2<T>(acc[d][nb][2] * mul, acc[d][nb][3] * mul);
-          if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(outp + 16 * d + 4 * q4) = w;
+          if (16 * d + 4 * q4 < width) *reinterpret_cast<i32x2*>(outp + 16 * d + 4 * q4) = w;
         }
       }
     }
@@ -460,9 +461,9 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
 
   using Loader = AsyncTileLoader<HD, BM, 256>;
   Loader ld;
-  ld.init(tid, a.D);
-  ld.load(Qs, a.q + b * a.sq.b + hkv * a.sq.h, a.sq.t, r0, r_end);
-  ld.load(dOs, a.d_o + b * a.sdo.b + hkv * a.sdo.h, a.sdo.t, r0, r_end);
+  ld.init(tid);
+  ld.load(Qs, a.q + b * a.sq.b + hkv * a.sq.h, a.sq.t, r0, r_end, a.D);
+  ld.load(dOs, a.d_o + b * a.sdo.b + hkv * a.sdo.h, a.sdo.t, r0, r_end, a.Dv);
   if (tid < BM) {
     const int r = r0 + tid;
     const bool in = r < r_end;
@@ -480,14 +481,15 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
   const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
   const int prow = lane / CH, pch = lane % CH;  // this lane's row within a pass over the private tile, its physical chunk
   WaveTileLoader<HD> own;
-  own.init(lane, a.D);
-  // columns [cb, cb + 32) of a depth tensor -> the private tile (rows past the chunk's last column arrive as zeros)
+  own.init(lane);
+  // columns [cb, cb + 32) of a depth tensor of head dim d -> the private tile (rows past the chunk's last column
+  // arrive as zeros)
   const bool partial = a.Lv != a.L;
-  auto fetch = [&](const uint16_t* base, int64_t stride, int cb) {
+  auto fetch = [&](const uint16_t* base, int64_t stride, int cb, int d) {
     if (partial)
-      own.fetch_mapped(wt, base, stride, cb, min(32, c_end - cb), (int64_t)a.T * a.L, a.L, a.Lv);
+      own.fetch_mapped(wt, base, stride, cb, min(32, c_end - cb), (int64_t)a.T * a.L, a.L, a.Lv, d);
     else
-      own.fetch(wt, base, stride, cb, min(32, c_end - cb));
+      own.fetch(wt, base, stride, cb, min(32, c_end - cb), d);
   };
   auto landed = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
@@ -499,7 +501,7 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
     asm volatile("" ::: "memory");
   };
   // 32 gradient rows from the accumulators (one column per lane) through the private tile to global memory
-  auto store = [&](const f32x16 (&acc)[DB], uint16_t* base, int64_t stride, int cb, float mul) {
+  auto store = [&](const f32x16 (&acc)[DB], uint16_t* base, int64_t stride, int cb, float mul, int width) {
     reads_done();
 #pragma unroll
     for (int d = 0; d < DB; d++)
@@ -515,7 +517,7 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
       const int row = i * RPW + prow;
       i32x4 val = *reinterpret_cast<MODA_LDS const i32x4*>(wt + i * 512 + lane * 8);
       const int lch = pch ^ Tile<HD>::swz(row);
-      if (cb + row < c_end && lch * 8 < a.D) {
+      if (cb + row < c_end && lch * 8 < width) {
         i32x4* dst = reinterpret_cast<i32x4*>(base + depth_row_of(a, cb + row) * stride + lch * 8);
         if (a.accum_depth) {  // add to what the row holds (this lane is the only writer of its 16 bytes)
           const i32x4 old = *dst;
@@ -537,13 +539,13 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
     // the column's visible rows: from its owner token's first row to the end of the chunk
     const int qlo = c < c_end ? (c / a.Lv) * a.Gf : r_end;
     reads_done();
-    fetch(kdp, a.skd.t, cb);
+    fetch(kdp, a.skd.t, cb, a.D);
     landed();
     i32x4 Sr[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) Sr[kk] = oa.row_operand(wt, 0, kk);
     reads_done();
-    fetch(vdp, a.svd.t, cb);  // the V rows travel while the probabilities are computed
+    fetch(vdp, a.svd.t, cb, a.Dv);  // the V rows travel while the probabilities are computed
     // S = Q K^T, P = exp2(S c - lse) on the visible rows
     f32x16 s[2];
     mfma_rows<T, HD, 2, 4>(oa, Qs, Sr, s);
@@ -575,7 +577,7 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
       TrPipe<T, HD, 4, 2> dvp;
       dvp.prefetch(oa, dOs);
       dvp.run(oa, dOs, P, acc);
-      store(acc, a.dvd + b * a.sdvd.b + hkv * a.sdvd.h, a.sdvd.t, cb, 1.f);
+      store(acc, a.dvd + b * a.sdvd.b + hkv * a.sdvd.h, a.sdvd.t, cb, 1.f, a.Dv);
     }
     {  // dP - delta = dO V^T (accumulators start from minus delta), dS = P (dP - delta), dK^T = Q^T dS
       f32x16 dp[2];
@@ -607,7 +609,7 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
       TrPipe<T, HD, 4, 2> dkp;
       dkp.prefetch(oa, Qs);
       dkp.run(oa, Qs, DS, acc);
-      store(acc, a.dkd + b * a.sdkd.b + hkv * a.sdkd.h, a.sdkd.t, cb, a.scale);
+      store(acc, a.dkd + b * a.sdkd.b + hkv * a.sdkd.h, a.sdkd.t, cb, a.scale, a.D);
     }
   }
 }
@@ -656,23 +658,24 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   const int w = (int)(c / a.L), slot = (int)(c - (int64_t)w * a.L);
   uint16_t* dk_out = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + c * a.sdkd.t + 8 * sub;
   uint16_t* dv_out = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + c * a.sdvd.t + 8 * sub;
-  const bool in_dim = 8 * sub < a.D;  // lanes past the tensors' head dim carry zeros and store nothing
+  // lanes past a tensor's head dim carry zeros and store nothing (keys and values may differ in width)
+  const bool in_k = 8 * sub < a.D, in_v = 8 * sub < a.Dv;
   if (slot >= a.Lv) {  // a slot without data: zero gradient, or (accumulating) somebody else's sum to leave alone
-    if (a.accum_depth || !in_dim) return;
+    if (a.accum_depth) return;
     const i32x4 z = {0, 0, 0, 0};
-    *reinterpret_cast<i32x4*>(dk_out) = z;
-    *reinterpret_cast<i32x4*>(dv_out) = z;
+    if (in_k) *reinterpret_cast<i32x4*>(dk_out) = z;
+    if (in_v) *reinterpret_cast<i32x4*>(dv_out) = z;
     return;
   }
-  auto load8 = [&](const uint16_t* p, float (&f)[8]) {
+  auto load8 = [&](const uint16_t* p, float (&f)[8], bool in_dim) {
     const i32x4 zero = {0, 0, 0, 0};
     const i32x4 v = in_dim ? *reinterpret_cast<const i32x4*>(p) : zero;
 #pragma unroll
     for (int i = 0; i < 4; i++) unpack2<T>(v[i], f[2 * i], f[2 * i + 1]);
   };
   float kf[8], vf[8], dk[8], dv[8];
-  load8(a.kd + b * a.skd.b + hkv * a.skd.h + c * a.skd.t + 8 * sub, kf);
-  load8(a.vd + b * a.svd.b + hkv * a.svd.h + c * a.svd.t + 8 * sub, vf);
+  load8(a.kd + b * a.skd.b + hkv * a.skd.h + c * a.skd.t + 8 * sub, kf, in_k);
+  load8(a.vd + b * a.svd.b + hkv * a.svd.h + c * a.svd.t + 8 * sub, vf, in_v);
 #pragma unroll
   for (int i = 0; i < 8; i++) dk[i] = dv[i] = 0.f;
   const float sc = a.scale * kLog2e;
@@ -681,8 +684,8 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   for (int gq = 0; gq < a.Gf; gq++) {
     const int64_t r = (int64_t)w * a.Gf + gq;
     float qf[8], dof[8];
-    load8(qb + r * a.sq.t, qf);
-    load8(dob + r * a.sdo.t, dof);
+    load8(qb + r * a.sq.t, qf, in_k);
+    load8(dob + r * a.sdo.t, dof, in_v);
     float s = 0.f, dp = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -706,8 +709,8 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   for (int i = 0; i < 8; i++) dk[i] *= a.scale;
   if (a.accum_depth) {  // add to what the row holds (this thread is its only writer), one rounding per call
     float ok_old[8], ov_old[8];
-    load8(dk_out, ok_old);
-    load8(dv_out, ov_old);
+    load8(dk_out, ok_old, in_k);
+    load8(dv_out, ov_old, in_v);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       dk[i] += ok_old[i];
@@ -720,10 +723,8 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
     ok[i] = pack2<T>(dk[2 * i], dk[2 * i + 1]);
     ov[i] = pack2<T>(dv[2 * i], dv[2 * i + 1]);
   }
-  if (in_dim) {
-    *reinterpret_cast<i32x4*>(dk_out) = ok;
-    *reinterpret_cast<i32x4*>(dv_out) = ov;
-  }
+  if (in_k) *reinterpret_cast<i32x4*>(dk_out) = ok;
+  if (in_v) *reinterpret_cast<i32x4*>(dv_out) = ov;
 }
 
 // Chunk-visible mode with a partially filled depth stream, not accumulating: the kernels above only visit the slots
@@ -739,10 +740,10 @@ __global__ __launch_bounds__(256) void zero_unfilled_slots_kernel(const KArgs a,
   rest /= a.Hkv;
   const int64_t row = rest % rows;
   const int64_t b = rest / rows;
-  if (b >= batches || 8 * sub >= a.D || (int)(row % a.L) < a.Lv) return;
+  if (b >= batches || (int)(row % a.L) < a.Lv) return;
   const i32x4 z = {0, 0, 0, 0};
-  *reinterpret_cast<i32x4*>(a.dkd + b * a.sdkd.b + h * a.sdkd.h + row * a.sdkd.t + 8 * sub) = z;
-  *reinterpret_cast<i32x4*>(a.dvd + b * a.sdvd.b + h * a.sdvd.h + row * a.sdvd.t + 8 * sub) = z;
+  if (8 * sub < a.D) *reinterpret_cast<i32x4*>(a.dkd + b * a.sdkd.b + h * a.sdkd.h + row * a.sdkd.t + 8 * sub) = z;
+  if (8 * sub < a.Dv) *reinterpret_cast<i32x4*>(a.dvd + b * a.sdvd.b + h * a.sdvd.h + row * a.sdvd.t + 8 * sub) = z;
 }
 
 // Adds the fp32 partial sums of the row segments (in segment order: the result does not depend on which
@@ -779,7 +780,7 @@ __global__ __launch_bounds__(256) void dkv_reduce_kernel(const KArgs a) {
     for (int i = 0; i < 4; i++) w[i] = pack2<T>(s[2 * i], s[2 * i + 1]);
     uint16_t* outp = which == 0 ? a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t
                                 : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t;
-    if (8 * sub < a.D) *reinterpret_cast<i32x4*>(outp + 8 * sub) = w;
+    if (8 * sub < (which == 0 ? a.D : a.Dv)) *reinterpret_cast<i32x4*>(outp + 8 * sub) = w;
   }
 }
 

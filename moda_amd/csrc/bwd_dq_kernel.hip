@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a_in) {
   const int r = rb * RPB + tid / TPR;
   const int c = (tid % TPR) * 8;
   float acc = 0.f;
-  if (r < a.Tq && c < a.D) {
+  if (r < a.Tq && c < a.Dv) {
     const uint16_t* op = a.o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + c;
     const uint16_t* dp = a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + c;
     const typename T::vec8 ov = *reinterpret_cast<const typename T::vec8*>(op);
@@ -90,9 +90,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       i32x4 z = {0, 0, 0, 0};
-      const bool in = valid && 32 * ks + 8 * q4 < a.D;
-      Qr[nb][ks] = in ? *reinterpret_cast<const i32x4*>(qp + 32 * ks) : z;
-      dOr[nb][ks] = in ? *reinterpret_cast<const i32x4*>(dop + 32 * ks) : z;
+      Qr[nb][ks] = (valid && 32 * ks + 8 * q4 < a.D) ? *reinterpret_cast<const i32x4*>(qp + 32 * ks) : z;
+      dOr[nb][ks] = (valid && 32 * ks + 8 * q4 < a.Dv) ? *reinterpret_cast<const i32x4*>(dop + 32 * ks) : z;
     }
     lse[nb] = 0.f;
     delta[nb] = 0.f;
@@ -129,30 +128,31 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   typedef AsyncTileLoader<HD, BN, NT, DMA_NOP> Loader;
   constexpr int LPT = 2 * Loader::N;
   Loader ld;
-  ld.init(tid, a.D);
+  ld.init(tid);
   typename Loader::Source srcK, srcV;
   if (a.has_seq && n_seq > 0) {
-    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
-    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
+    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T, a.D);
+    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T, a.Dv);
   }
   int ld_st = 0;
   auto issue = [&](int it) {
     lds_ptr Kt = smem + ld_st * 2 * BN * HD;
     if (!NODEPTH && it == n_seq) {
-      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
-      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
+      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L, a.D);
+      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L, a.Dv);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
     if (PARTIAL && it >= n_seq) {  // depth tile of a partially filled stream: rows through the slot mapping
-      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
-      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
+      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv, a.D);
+      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv,
+                     a.Dv);
     } else if (WIDE) {
       const bool dep = !NODEPTH && it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
-              row0, row_end);
+              row0, row_end, a.D);
       ld.load(Kt + BN * HD, dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h,
-              dep ? a.svd.t : a.sv.t, row0, row_end);
+              dep ? a.svd.t : a.sv.t, row0, row_end, a.Dv);
     } else {
       ld.load_from(Kt, srcK, row0);
       ld.load_from(Kt + BN * HD, srcV, row0);
@@ -268,17 +268,17 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
       const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
       const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
       Own own;
-      own.init(lane, a.D);
-      // rows [col0, col0 + 32) of the span (short at its end) into a private tile
-      auto fetch = [&](lds_ptr tile, const uint16_t* slice, int64_t stride, int col0) {
+      own.init(lane);
+      // rows [col0, col0 + 32) of the span (short at its end) into a private tile; d: the tensor's head dim
+      auto fetch = [&](lds_ptr tile, const uint16_t* slice, int64_t stride, int col0, int d) {
         const int nrows = min(32, c_end - col0);
         if (PARTIAL)
-          own.fetch_mapped(tile, slice, stride, col0, nrows, (int64_t)a.T * a.L, a.L, a.Lv);
+          own.fetch_mapped(tile, slice, stride, col0, nrows, (int64_t)a.T * a.L, a.L, a.Lv, d);
         else
-          own.fetch(tile, slice, stride, col0, nrows);
+          own.fetch(tile, slice, stride, col0, nrows, d);
       };
-      fetch(Kt, kdp, a.skd.t, c_beg);
-      fetch(Vt, vdp, a.svd.t, c_beg);
+      fetch(Kt, kdp, a.skd.t, c_beg, a.D);
+      fetch(Vt, vdp, a.svd.t, c_beg, a.Dv);
       const std::integral_constant<int, 2> two{};
       for (int j = 0; j < nh; j++) {
         const int col0 = c_beg + 32 * j;
@@ -286,10 +286,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
         Own::template wait_but<0>();
         tile(std::true_type{}, two, Kt, Vt, col0, dlo, dhi, [&]() {
           Own::reads_done();
-          if (more) fetch(Vt, vdp, a.svd.t, col0 + 32);
+          if (more) fetch(Vt, vdp, a.svd.t, col0 + 32, a.Dv);
         });
         Own::reads_done();
-        if (more) fetch(Kt, kdp, a.skd.t, col0 + 32);
+        if (more) fetch(Kt, kdp, a.skd.t, col0 + 32, a.D);
       }
     }
   }

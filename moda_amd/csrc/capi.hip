@@ -52,16 +52,18 @@ int value_dim(const moda_hip_desc* d) { return (int)(d->Dv > 0 ? d->Dv : d->D); 
 // 16-byte chunks) up to 256 runs on the next width, zero-padded inside the kernels.
 bool mfma_shape(const moda_hip_desc* d) {
   return (d->dtype == MODA_HIP_BF16 || d->dtype == MODA_HIP_FP16) && d->D % 8 == 0 && d->D <= 256 &&
-         value_dim(d) == d->D;
+         value_dim(d) % 8 == 0 && value_dim(d) <= 256;
 }
 // Packed variable-length batches with head dims above 128 do not run the packed instantiations of the 256-wide
 // kernels: that combination (with chunk-visible mode) once ended in a GPU memory fault whose cause was never
 // found, so those instantiations stay switched off.  With a host copy of the offsets the batch runs as one launch
 // per sequence on the fixed-length 256-wide kernels (per_sequence below); without it, on the vector-ALU kernels.
-bool packed_wide(const moda_hip_desc* d) { return d->D > 128 && d->cu_seqlens; }
+int widest_dim(const moda_hip_desc* d) { return (int)(d->D > value_dim(d) ? d->D : value_dim(d)); }
+bool packed_wide(const moda_hip_desc* d) { return widest_dim(d) > 128 && d->cu_seqlens; }
 bool per_sequence(const moda_hip_desc* d) { return mfma_shape(d) && packed_wide(d) && d->cu_seqlens_host; }
 bool use_mfma(const moda_hip_desc* d) { return mfma_shape(d) && !packed_wide(d); }
-int tile_width(const moda_hip_desc* d) { return d->D <= 64 ? 64 : d->D <= 128 ? 128 : 256; }
+// keys and values share one tile width: that of the wider of the two head dims
+int tile_width(const moda_hip_desc* d) { return widest_dim(d) <= 64 ? 64 : widest_dim(d) <= 128 ? 128 : 256; }
 
 // Validates the descriptor and fills the geometry part of KArgs.
 int fill_geometry(const moda_hip_desc* d, KArgs& a) {
@@ -86,6 +88,7 @@ int fill_geometry(const moda_hip_desc* d, KArgs& a) {
   a.T = (int)d->T;
   a.Hkv = (int)d->H;
   a.D = (int)d->D;
+  a.Dv = value_dim(d);
   a.Tq = plain ? (int)d->T : (int)(d->T * d->G);
   a.Gf = plain ? 1 : (int)d->G;
   a.Hq = plain ? (int)(d->H * d->G) : (int)d->H;
@@ -134,7 +137,7 @@ size_t delta_bytes(const KArgs& a) { return (delta_bytes_exact(a) + 255) / 256 *
 // partition mode, so that the workspace size depends on the descriptor alone.
 int desired_dkv_split(const moda_hip_desc* d, const KArgs& a) {
   if (!use_mfma(d) || a.cu || !a.has_seq || a.T == 0) return 1;
-  const int cols = d->D > 128 ? 64 : 128, rows = d->D > 128 ? 32 : 64;  // the kernel's column tile and query tile
+  const int cols = widest_dim(d) > 128 ? 64 : 128, rows = widest_dim(d) > 128 ? 32 : 64;  // the kernel's column tile and query tile
   const int64_t tiles = (int64_t)((a.T + cols - 1) / cols) * a.B * a.Hkv;
   const int64_t query_tiles = (a.Tq + rows - 1) / rows;
   int s = 1;

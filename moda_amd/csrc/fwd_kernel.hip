@@ -99,32 +99,33 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   typedef AsyncTileLoader<HD, BN, NT> Loader;
   constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
   Loader ld;
-  ld.init(tid, a.D);
+  ld.init(tid);
   // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
   // producer reaches the first depth tile
   typename Loader::Source srcK, srcV;
   if (a.has_seq && n_seq > 0) {
-    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
-    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
+    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T, a.D);
+    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T, a.Dv);
   }
   int ld_st = 0;  // ring stage the next issued tile goes to
   auto issue = [&](int it) {
     lds_ptr Kt = smem + ld_st * 2 * BN * HD;
     if (!NODEPTH && it == n_seq) {
-      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
-      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
+      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L, a.D);
+      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L, a.Dv);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
     if (PARTIAL && it >= n_seq) {  // depth tile of a partially filled stream: rows through the slot mapping
-      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
-      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
+      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv, a.D);
+      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv,
+                     a.Dv);
     } else if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
       const bool dep = !NODEPTH && it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
-              row0, row_end);
+              row0, row_end, a.D);
       ld.load(Kt + BN * HD, dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h,
-              dep ? a.svd.t : a.sv.t, row0, row_end);
+              dep ? a.svd.t : a.sv.t, row0, row_end, a.Dv);
     } else {
       ld.load_from(Kt, srcK, row0);
       ld.load_from(Kt + BN * HD, srcV, row0);
@@ -346,17 +347,17 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
       const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
       const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
       Own own;
-      own.init(lane, a.D);
-      // rows [col0, col0 + 32) of the span (short at its end) into a private tile
-      auto fetch = [&](lds_ptr tile, const uint16_t* slice, int64_t stride, int col0) {
+      own.init(lane);
+      // rows [col0, col0 + 32) of the span (short at its end) into a private tile; d: the tensor's head dim
+      auto fetch = [&](lds_ptr tile, const uint16_t* slice, int64_t stride, int col0, int d) {
         const int nrows = min(32, c_end - col0);
         if (PARTIAL)
-          own.fetch_mapped(tile, slice, stride, col0, nrows, (int64_t)a.T * a.L, a.L, a.Lv);
+          own.fetch_mapped(tile, slice, stride, col0, nrows, (int64_t)a.T * a.L, a.L, a.Lv, d);
         else
-          own.fetch(tile, slice, stride, col0, nrows);
+          own.fetch(tile, slice, stride, col0, nrows, d);
       };
-      fetch(Kt, kdp, a.skd.t, c_beg);
-      fetch(Vt, vdp, a.svd.t, c_beg);
+      fetch(Kt, kdp, a.skd.t, c_beg, a.D);
+      fetch(Vt, vdp, a.svd.t, c_beg, a.Dv);
       const std::integral_constant<int, 1> one{};
       for (int j = 0; j < nh; j++) {
         const int col0 = c_beg + 32 * j;
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         Own::template wait_but<Own::N>();  // K landed, V may still be on its way
         front(std::true_type{}, one, Kt, col0, dlo, dhi, []() {});
         Own::reads_done();
-        if (more) fetch(Kt, kdp, a.skd.t, col0 + 32);
+        if (more) fetch(Kt, kdp, a.skd.t, col0 + 32, a.D);
         if (more)
           Own::template wait_but<Own::N>();  // V landed, the next K on its way
         else
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         pv1.prefetch(oa, Vt);
         pv1.run(oa, Vt, P1, o);
         Own::reads_done();
-        if (more) fetch(Vt, vdp, a.svd.t, col0 + 32);
+        if (more) fetch(Vt, vdp, a.svd.t, col0 + 32, a.Dv);
       }
     }
   }
@@ -389,7 +390,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         i32x2 w;
         w[0] = pack2<T>(o[d][4 * i4 + 0] * inv, o[d][4 * i4 + 1] * inv);
         w[1] = pack2<T>(o[d][4 * i4 + 2] * inv, o[d][4 * i4 + 3] * inv);
-        if (32 * d + 8 * i4 + 4 * g < a.D) *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
+        if (32 * d + 8 * i4 + 4 * g < a.Dv) *reinterpret_cast<i32x2*>(op + 32 * d + 8 * i4 + 4 * g) = w;
       }
     if (g == 0) a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq] = (l > 0.f) ? m + log2f(l) : kNegInf;
   }
@@ -461,32 +462,33 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
   typedef AsyncTileLoader<HD, BN, NT> Loader;
   constexpr int LPT = 2 * Loader::N;  // vector-memory loads one wave issues per tile (K + V)
   Loader ld;
-  ld.init(tid, a.D);
+  ld.init(tid);
   // the two sources being streamed: sequence K/V first, swapped for the depth K/V when the
   // producer reaches the first depth tile
   typename Loader::Source srcK, srcV;
   if (a.has_seq && n_seq > 0) {
-    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
-    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
+    srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T, a.D);
+    srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T, a.Dv);
   }
   int ld_st = 0;  // ring stage the next issued tile goes to
   auto issue = [&](int it) {
     lds_ptr Kt = smem + ld_st * 2 * BN * HD;
     if (it == n_seq) {
-      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L);
-      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L);
+      srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, dep0, a.T * a.L, a.D);
+      srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, dep0, a.T * a.L, a.Dv);
     }
     const int row0 = it < n_seq ? it * BN : dep0 + (it - n_seq) * BN;
     if (PARTIAL && it >= n_seq) {  // depth tile of a partially filled stream: rows through the slot mapping
-      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
-      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv);
+      ld.load_mapped(Kt, a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv, a.D);
+      ld.load_mapped(Kt + BN * HD, a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, row0, (int64_t)a.T * a.L, a.L, a.Lv,
+                     a.Dv);
     } else if (WIDE) {  // some slice spans more than 2 GiB: a descriptor anchored at this tile
       const bool dep = it >= n_seq;
       const int row_end = dep ? a.T * a.L : a.T;
       ld.load(Kt, dep ? a.kd + b * a.skd.b + hkv * a.skd.h : a.k + b * a.sk.b + hkv * a.sk.h, dep ? a.skd.t : a.sk.t,
-              row0, row_end);
+              row0, row_end, a.D);
       ld.load(Kt + BN * HD, dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h,
-              dep ? a.svd.t : a.sv.t, row0, row_end);
+              dep ? a.svd.t : a.sv.t, row0, row_end, a.Dv);
     } else {
       ld.load_from(Kt, srcK, row0);
       ld.load_from(Kt + BN * HD, srcV, row0);
@@ -650,7 +652,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
         i32x2 w;
         w[0] = pack2<T>(o[d][nb][0] * inv, o[d][nb][1] * inv);
         w[1] = pack2<T>(o[d][nb][2] * inv, o[d][nb][3] * inv);
-        if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(op + 16 * d + 4 * q4) = w;
+        if (16 * d + 4 * q4 < a.Dv) *reinterpret_cast<i32x2*>(op + 16 * d + 4 * q4) = w;
       }
       if (q4 == 0) a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq] = (lsum > 0.f) ? m[nb] + log2f(lsum) : kNegInf;
     }

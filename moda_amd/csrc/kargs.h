@@ -16,7 +16,8 @@ struct KArgs {
   float* delta;        // [B, Hq, delta_pitch]   workspace: MINUS rowsum(o * do)
   Str3 sq, sk, sv, skd, svd, so, sdo, sdq, sdk, sdv, sdkd, sdvd;
   int B, T, Hkv;
-  int D;     // head dim of the tensors; the matrix kernels run it zero-padded to their tile width (64 or 128)
+  int D;     // head dim of q, k, kd and their gradients; the matrix kernels run it zero-padded to their tile width
+  int Dv;    // head dim of v, vd, o, do and their gradients (same tile width)
   int Tq;    // query rows per (batch, query head)
   int Gf;    // query rows per token (fold factor)
   int Hq;    // query-head programs per batch

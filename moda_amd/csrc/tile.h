@@ -384,8 +384,7 @@ struct AsyncTileLoader {
   int gchunk;       // logical chunk this lane fetches
   int wave;
 
-  // `d`: head dim of the tensors, a multiple of 8 not above HD
-  __host__ __device__ __forceinline__ void init(int tid, int d = HD) {
+  __host__ __device__ __forceinline__ void init(int tid) {
     const int lane = tid & 63;
 #if defined(__HIP_DEVICE_COMPILE__)
     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -394,11 +393,13 @@ struct AsyncTileLoader {
 #endif
     row_in_pass = wave * RPW + lane / CH;
     gchunk = (lane % CH) ^ Tile<HD>::swz(row_in_pass);
-    if (gchunk * 8 >= d) gchunk = -1;
   }
-  // this lane's byte offset inside a tile whose rows are `stride_bytes` apart
-  __host__ __device__ __forceinline__ int lane_offset(int stride_bytes) const {
-    return gchunk < 0 ? kPadOffset : row_in_pass * stride_bytes + gchunk * 16;
+  // whether this lane's chunk lies past a tensor's head dim `d` (a multiple of 8 not above HD): such lanes fetch
+  // out of range and receive zeros
+  __host__ __device__ __forceinline__ bool pads(int d) const { return gchunk * 8 >= d; }
+  // this lane's byte offset inside a tile of a tensor of head dim `d` whose rows are `stride_bytes` apart
+  __host__ __device__ __forceinline__ int lane_offset(int stride_bytes, int d) const {
+    return pads(d) ? kPadOffset : row_in_pass * stride_bytes + gchunk * 16;
   }
   // the i-th of a wave's N loads of a tile: element offset of the 64 LDS slots it fills, tile rows it skips
   __host__ __device__ __forceinline__ int lds_elems(int i) const { return (i * NW + wave) * 512; }
@@ -413,14 +414,15 @@ struct AsyncTileLoader {
     int stride_bytes;
     int row_base;
   };
-  __host__ __device__ __forceinline__ Source source(const uint16_t* slice, int64_t row_stride, int row_base, int row_end) const {
+  __host__ __device__ __forceinline__ Source source(const uint16_t* slice, int64_t row_stride, int row_base, int row_end,
+                                                    int d) const {
     Source s;
     s.stride_bytes = (int)row_stride * 2;
     s.row_base = row_base;
     const int64_t nbytes = (int64_t)(row_end > row_base ? row_end - row_base : 0) * s.stride_bytes;
     s.base = slice + (int64_t)row_base * row_stride;
     s.nbytes = nbytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)nbytes;
-    s.voff = lane_offset(s.stride_bytes);
+    s.voff = lane_offset(s.stride_bytes, d);
     return s;
   }
   // rows [row0, row0 + ROWS) of the source into `tile`; rows past the source's end arrive as zeros
@@ -439,28 +441,28 @@ struct AsyncTileLoader {
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     return rows_left <= 0 ? 0u : (uint32_t)(rows_left < ROWS ? rows_left : ROWS) * stride_bytes;
   }
-  __device__ __forceinline__ void load(lds_ptr tile, const uint16_t* src, int64_t row_stride, int row0,
-                                       int row_end) const {
+  __device__ __forceinline__ void load(lds_ptr tile, const uint16_t* src, int64_t row_stride, int row0, int row_end,
+                                       int d) const {
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const i32x4 rs = rsrc_words(src + (int64_t)row0 * row_stride, anchored_bytes(row_stride, row0, row_end));
-    const int voff = lane_offset((int)stride_bytes);
+    const int voff = lane_offset((int)stride_bytes, d);
 #pragma unroll
     for (int i = 0; i < N; i++) lds_dma<16, NOP>(rs, lds_addr(tile + lds_elems(i)), voff, rows_before(i) * (int)stride_bytes);
   }
   // this lane's byte offset, relative to the anchor, in load i of a mapped depth tile (see mapped_row)
-  __host__ __device__ __forceinline__ int mapped_offset(int i, int l0, int L, int Lv, int stride_bytes) const {
-    return gchunk < 0 ? kPadOffset : mapped_row(l0, rows_before(i) + row_in_pass, L, Lv) * stride_bytes + gchunk * 16;
+  __host__ __device__ __forceinline__ int mapped_offset(int i, int l0, int L, int Lv, int stride_bytes, int d) const {
+    return pads(d) ? kPadOffset : mapped_row(l0, rows_before(i) + row_in_pass, L, Lv) * stride_bytes + gchunk * 16;
   }
   // compact depth columns [col0, col0 + ROWS) of a slice of rows_total rows with L slots per token, Lv of them filled
   __device__ __forceinline__ void load_mapped(lds_ptr tile, const uint16_t* slice, int64_t row_stride, int col0,
-                                              int64_t rows_total, int L, int Lv) const {
+                                              int64_t rows_total, int L, int Lv, int d) const {
     const int w0 = __builtin_amdgcn_readfirstlane(col0 / Lv), l0 = col0 - w0 * Lv;
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const int64_t anchor = (int64_t)w0 * L;
     const i32x4 rs = rsrc_words(slice + anchor * row_stride, mapped_bytes(anchor, rows_total, stride_bytes));
 #pragma unroll
     for (int i = 0; i < N; i++)
-      lds_dma<16, NOP>(rs, lds_addr(tile + lds_elems(i)), mapped_offset(i, l0, L, Lv, (int)stride_bytes), 0);
+      lds_dma<16, NOP>(rs, lds_addr(tile + lds_elems(i)), mapped_offset(i, l0, L, Lv, (int)stride_bytes, d), 0);
   }
   // s_waitcnt vmcnt(0): every outstanding vector-memory load of this wave has landed
   __device__ __forceinline__ static void wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -478,42 +480,41 @@ struct AsyncTileLoader {
 template <int HD, int NOP = MODA_DMA_NOP>
 struct WaveTileLoader {
   static constexpr int CH = HD / 8, RPW = 64 / CH, N = 32 / RPW;  // chunks per row, rows per load, loads per tile
-  int prow, pch, d;
-  __host__ __device__ __forceinline__ void init(int lane, int head_dim) {
+  int prow, pch;
+  __host__ __device__ __forceinline__ void init(int lane) {
     prow = lane / CH;
     pch = lane % CH;
-    d = head_dim;
   }
-  // this lane's byte offset in load i of a tile (rows `stride_bytes` apart): its tile row is i * RPW + prow
-  __host__ __device__ __forceinline__ int lane_offset(int i, int stride_bytes) const {
+  // this lane's byte offset in load i of a tile (rows `stride_bytes` apart, head dim `d`): its tile row is i * RPW + prow
+  __host__ __device__ __forceinline__ int lane_offset(int i, int stride_bytes, int d) const {
     const int row = i * RPW + prow;
     const int lch = pch ^ Tile<HD>::swz(row);
     return lch * 8 < d ? row * stride_bytes + lch * 16 : kPadOffset;
   }
   // rows [row0, row0 + nrows) of the slice at `base` (nrows <= 32; the rest of the tile arrives as zeros)
-  __device__ __forceinline__ void fetch(lds_ptr tile, const uint16_t* base, int64_t row_stride, int64_t row0,
-                                        int nrows) const {
+  __device__ __forceinline__ void fetch(lds_ptr tile, const uint16_t* base, int64_t row_stride, int64_t row0, int nrows,
+                                        int d) const {
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const i32x4 rs = rsrc_words(base + row0 * row_stride, nrows > 0 ? (uint32_t)nrows * stride_bytes : 0u);
 #pragma unroll
-    for (int i = 0; i < N; i++) lds_dma<16, NOP>(rs, lds_addr(tile + i * 512), lane_offset(i, (int)stride_bytes), 0);
+    for (int i = 0; i < N; i++) lds_dma<16, NOP>(rs, lds_addr(tile + i * 512), lane_offset(i, (int)stride_bytes, d), 0);
   }
   // the same for a mapped depth tile (see mapped_row): offset relative to the anchor, rows >= nrows padded
-  __host__ __device__ __forceinline__ int mapped_offset(int i, int l0, int L, int Lv, int nrows, int stride_bytes) const {
+  __host__ __device__ __forceinline__ int mapped_offset(int i, int l0, int L, int Lv, int nrows, int stride_bytes, int d) const {
     const int row = i * RPW + prow;
     const int lch = pch ^ Tile<HD>::swz(row);
     return (lch * 8 < d && row < nrows) ? mapped_row(l0, row, L, Lv) * stride_bytes + lch * 16 : kPadOffset;
   }
   // compact depth columns [col0, col0 + nrows) of a slice of rows_total rows, L slots per token, Lv of them filled
   __device__ __forceinline__ void fetch_mapped(lds_ptr tile, const uint16_t* slice, int64_t row_stride, int col0,
-                                               int nrows, int64_t rows_total, int L, int Lv) const {
+                                               int nrows, int64_t rows_total, int L, int Lv, int d) const {
     const int w0 = __builtin_amdgcn_readfirstlane(col0 / Lv), l0 = col0 - w0 * Lv;
     const uint32_t stride_bytes = (uint32_t)row_stride * 2u;
     const int64_t anchor = (int64_t)w0 * L;
     const i32x4 rs = rsrc_words(slice + anchor * row_stride, nrows > 0 ? mapped_bytes(anchor, rows_total, stride_bytes) : 0u);
 #pragma unroll
     for (int i = 0; i < N; i++)
-      lds_dma<16, NOP>(rs, lds_addr(tile + i * 512), mapped_offset(i, l0, L, Lv, nrows, (int)stride_bytes), 0);
+      lds_dma<16, NOP>(rs, lds_addr(tile + i * 512), mapped_offset(i, l0, L, Lv, nrows, (int)stride_bytes, d), 0);
   }
   // at most K of this wave's vector-memory loads (the youngest) still in flight
   template <int K>

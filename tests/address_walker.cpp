@@ -18,7 +18,7 @@
 //     fills lie inside the launch's dynamic LDS allocation;
 //   * coverage: every element of o, lse, dq, dk, dv, dkd, dvd and of the row-sum workspace is written exactly once.
 //
-// usage: address_walker HD D H G L Lv mode(0..4) chunk_tokens hdiv_plain packed B_or_n len0 [len1 ...]
+// usage: address_walker HD D Dv H G L Lv mode(0..4) chunk_tokens row_segments packed B_or_n len0 [len1 ...]
 //   packed = 0: a fixed-length batch of B sequences of len0 tokens; packed = 1: n sequences on one packed axis.
 #include <hip/hip_runtime.h>
 
@@ -126,7 +126,7 @@ void check_dma(const char* name, const void* desc_base, uint32_t num_records, in
 }
 
 struct Case {
-  int HD, D, H, G, L, Lv, mode, cb, packed, nseq;
+  int HD, D, Dv, H, G, L, Lv, mode, cb, packed, nseq;
   std::vector<int> len;
   std::vector<int32_t> cu;
   int total, Tmax;
@@ -142,6 +142,7 @@ KArgs make_args(const Case& c) {
   a.T = c.Tmax;
   a.Hkv = c.H;
   a.D = c.D;
+  a.Dv = c.Dv;
   a.Tq = plain ? c.Tmax : c.Tmax * c.G;
   a.Gf = plain ? 1 : c.G;
   a.Hq = plain ? c.H * c.G : c.H;
@@ -157,28 +158,31 @@ KArgs make_args(const Case& c) {
   a.compute_units = 256;
   const int64_t qrows = plain ? T : (int64_t)T * c.G;
   a.delta_pitch = c.packed ? (int)qrows : a.Tq;
-  auto strides = [&](int64_t rows, int heads) { return Str3{rows * heads * c.D, (int64_t)heads * c.D, (int64_t)c.D}; };
-  const uint64_t qb = (uint64_t)Bt * qrows * a.Hq * c.D * 2, kb = (uint64_t)Bt * T * c.H * c.D * 2,
-                 db = (uint64_t)Bt * T * c.L * c.H * c.D * 2;
+  auto strides = [&](int64_t rows, int heads, int dim) { return Str3{rows * heads * dim, (int64_t)heads * dim, (int64_t)dim}; };
+  // bytes of a dense [Bt, rows, heads, dim] tensor of 16-bit elements
+  auto bytes = [&](int64_t rows, int heads, int dim) { return (uint64_t)Bt * rows * heads * dim * 2; };
   int idx = 0;
-  a.q = add_region("q", idx++, qb, 2, false);
-  a.o = add_region("o", idx++, qb, 2, true);
+  a.q = add_region("q", idx++, bytes(qrows, a.Hq, c.D), 2, false);
+  a.o = add_region("o", idx++, bytes(qrows, a.Hq, c.Dv), 2, true);
   a.out_o = (uint16_t*)a.o;
-  a.d_o = add_region("do", idx++, qb, 2, false);
-  a.dq = (uint16_t*)add_region("dq", idx++, qb, 2, true);
-  a.k = add_region("k", idx++, kb, 2, false);
-  a.v = add_region("v", idx++, kb, 2, false);
-  a.dk = (uint16_t*)add_region("dk", idx++, kb, 2, true);
-  a.dv = (uint16_t*)add_region("dv", idx++, kb, 2, true);
-  a.kd = add_region("kd", idx++, db, 2, false);
-  a.vd = add_region("vd", idx++, db, 2, false);
-  a.dkd = (uint16_t*)add_region("dkd", idx++, db, 2, true);
-  a.dvd = (uint16_t*)add_region("dvd", idx++, db, 2, true);
+  a.d_o = add_region("do", idx++, bytes(qrows, a.Hq, c.Dv), 2, false);
+  a.dq = (uint16_t*)add_region("dq", idx++, bytes(qrows, a.Hq, c.D), 2, true);
+  a.k = add_region("k", idx++, bytes(T, c.H, c.D), 2, false);
+  a.v = add_region("v", idx++, bytes(T, c.H, c.Dv), 2, false);
+  a.dk = (uint16_t*)add_region("dk", idx++, bytes(T, c.H, c.D), 2, true);
+  a.dv = (uint16_t*)add_region("dv", idx++, bytes(T, c.H, c.Dv), 2, true);
+  a.kd = add_region("kd", idx++, bytes((int64_t)T * c.L, c.H, c.D), 2, false);
+  a.vd = add_region("vd", idx++, bytes((int64_t)T * c.L, c.H, c.Dv), 2, false);
+  a.dkd = (uint16_t*)add_region("dkd", idx++, bytes((int64_t)T * c.L, c.H, c.D), 2, true);
+  a.dvd = (uint16_t*)add_region("dvd", idx++, bytes((int64_t)T * c.L, c.H, c.Dv), 2, true);
   a.lse = (float*)add_region("lse", idx++, (uint64_t)Bt * qrows * a.Hq * 4, 4, true);
   a.delta = (float*)add_region("delta", idx++, (uint64_t)(c.packed ? 1 : c.nseq) * a.Hq * a.delta_pitch * 4, 4, true);
-  a.sq = a.so = a.sdo = a.sdq = strides(qrows, a.Hq);
-  a.sk = a.sv = a.sdk = a.sdv = strides(T, c.H);
-  a.skd = a.svd = a.sdkd = a.sdvd = strides((int64_t)T * c.L, c.H);
+  a.sq = a.sdq = strides(qrows, a.Hq, c.D);
+  a.so = a.sdo = strides(qrows, a.Hq, c.Dv);
+  a.sk = a.sdk = strides(T, c.H, c.D);
+  a.sv = a.sdv = strides(T, c.H, c.Dv);
+  a.skd = a.sdkd = strides((int64_t)T * c.L, c.H, c.D);
+  a.svd = a.sdvd = strides((int64_t)T * c.L, c.H, c.Dv);
   if (c.packed) a.cu = c.cu.data();
   return a;
 }
@@ -233,9 +237,8 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
         const int step = rows_per_wave == 32 ? 16 : 32;
         ctx(kname, (int)block, wave, lane, "Q / dO register rows");
         for (int e = piece; e < HD; e += step) {
-          if (e >= a.D) continue;
-          check_access("q", a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + e, 16, false);
-          if (dq) check_access("do", a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + e, 16, false);
+          if (e < a.D) check_access("q", a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + e, 16, false);
+          if (dq && e < a.Dv) check_access("do", a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + e, 16, false);
         }
         const bool stat_lane = rows_per_wave == 32 ? (lane >> 5) == 0 : (lane >> 4) == 0;
         ctx(kname, (int)block, wave, lane, "row statistics and result rows");
@@ -248,28 +251,25 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
         // result row: 8-byte stores, lane group g / q4 owns elements 4g + 8j (32x32) or 4q + 16j (16x16)
         const int first = rows_per_wave == 32 ? 4 * (lane >> 5) : 4 * (lane >> 4), stride = rows_per_wave == 32 ? 8 : 16;
         for (int e = first; e < HD; e += stride) {
-          if (e >= a.D) continue;
-          if (dq)
-            check_access("dq", a.dq + b * a.sdq.b + hq * a.sdq.h + (int64_t)r * a.sdq.t + e, 8, true);
-          else
-            check_access("o", a.out_o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + e, 8, true);
+          if (dq && e < a.D) check_access("dq", a.dq + b * a.sdq.b + hq * a.sdq.h + (int64_t)r * a.sdq.t + e, 8, true);
+          if (!dq && e < a.Dv) check_access("o", a.out_o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + e, 8, true);
         }
       }
       // ring tiles: every tile 0 .. ntiles-1 is issued once, stages in turn
       Loader ld;
-      ld.init(tid, a.D);
+      ld.init(tid);
       typename Loader::Source srcK{}, srcV{};
       if (a.has_seq && plan.n_seq > 0) {
-        srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T);
-        srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T);
+        srcK = ld.source(a.k + b * a.sk.b + hkv * a.sk.h, a.sk.t, 0, a.T, a.D);
+        srcV = ld.source(a.v + b * a.sv.b + hkv * a.sv.h, a.sv.t, 0, a.T, a.Dv);
       }
       for (int it = 0; it < ntiles; it++) {
         const int st = it % NST;
         const uint32_t kt = (uint32_t)st * 2 * BN * HD * 2;
         const bool dep = it >= plan.n_seq;
         if (Ld > 0 && it == plan.n_seq) {
-          srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, plan.dep0, a.T * a.L);
-          srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, plan.dep0, a.T * a.L);
+          srcK = ld.source(a.kd + b * a.skd.b + hkv * a.skd.h, a.skd.t, plan.dep0, a.T * a.L, a.D);
+          srcV = ld.source(a.vd + b * a.svd.b + hkv * a.svd.h, a.svd.t, plan.dep0, a.T * a.L, a.Dv);
         }
         const int row0 = ring_tile_row0(plan, it, BN);
         ctx(kname, (int)block, wave, lane, dep ? "ring depth tile" : "ring sequence tile");
@@ -280,10 +280,10 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
             const int64_t anchor = (int64_t)w0 * a.L, rows_total = (int64_t)a.T * a.L;
             check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + anchor * a.skd.t,
                       mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u),
-                      ld.mapped_offset(i, l0, a.L, a.Lv, (int)a.skd.t * 2), 0, 16, ldsK, lds_bytes, ld.gchunk < 0);
+                      ld.mapped_offset(i, l0, a.L, a.Lv, (int)a.skd.t * 2, a.D), 0, 16, ldsK, lds_bytes, ld.pads(a.D));
             check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + anchor * a.svd.t,
                       mapped_bytes(anchor, rows_total, (uint32_t)a.svd.t * 2u),
-                      ld.mapped_offset(i, l0, a.L, a.Lv, (int)a.svd.t * 2), 0, 16, ldsV, lds_bytes, ld.gchunk < 0);
+                      ld.mapped_offset(i, l0, a.L, a.Lv, (int)a.svd.t * 2, a.Dv), 0, 16, ldsV, lds_bytes, ld.pads(a.Dv));
             // a lane in range must have fetched a slot that holds data
             const int rel = mapped_row(l0, Loader::rows_before(i) + ld.row_in_pass, a.L, a.Lv);
             if ((anchor + rel) % a.L >= a.Lv) fail("mapped depth tile reads slot %d of %d filled", (int)((anchor + rel) % a.L), a.Lv);
@@ -293,14 +293,14 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
             const uint16_t* vb = dep ? a.vd + b * a.svd.b + hkv * a.svd.h : a.v + b * a.sv.b + hkv * a.sv.h;
             const int64_t ks = dep ? a.skd.t : a.sk.t, vs = dep ? a.svd.t : a.sv.t;
             check_dma(dep ? "kd" : "k", kb + (int64_t)row0 * ks, Loader::anchored_bytes(ks, row0, row_end),
-                      ld.lane_offset((int)ks * 2), Loader::rows_before(i) * (int)ks * 2, 16, ldsK, lds_bytes, ld.gchunk < 0);
+                      ld.lane_offset((int)ks * 2, a.D), Loader::rows_before(i) * (int)ks * 2, 16, ldsK, lds_bytes, ld.pads(a.D));
             check_dma(dep ? "vd" : "v", vb + (int64_t)row0 * vs, Loader::anchored_bytes(vs, row0, row_end),
-                      ld.lane_offset((int)vs * 2), Loader::rows_before(i) * (int)vs * 2, 16, ldsV, lds_bytes, ld.gchunk < 0);
+                      ld.lane_offset((int)vs * 2, a.Dv), Loader::rows_before(i) * (int)vs * 2, 16, ldsV, lds_bytes, ld.pads(a.Dv));
           } else {
             check_dma(dep ? "kd" : "k", srcK.base, srcK.nbytes, srcK.voff, Loader::source_soffset(srcK, row0, i), 16, ldsK,
-                      lds_bytes, ld.gchunk < 0);
+                      lds_bytes, ld.pads(a.D));
             check_dma(dep ? "vd" : "v", srcV.base, srcV.nbytes, srcV.voff, Loader::source_soffset(srcV, row0, i), 16, ldsV,
-                      lds_bytes, ld.gchunk < 0);
+                      lds_bytes, ld.pads(a.Dv));
           }
         }
       }
@@ -313,7 +313,7 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
           const DepthSpan span = own_depth_span(a, rw0, rows_per_wave);
           const int nh = (span.c_end - span.c_beg + 31) / 32;
           Own own;
-          own.init(lane, a.D);
+          own.init(lane);
           ctx(kname, (int)block, wave, lane, "own depth tile");
           for (int j = 0; j < nh; j++) {
             const int col0 = span.c_beg + 32 * j;
@@ -322,8 +322,8 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
               if (a.Lv != a.L) {
                 const int w0 = col0 / a.Lv, l0 = col0 - w0 * a.Lv;
                 const int64_t anchor = (int64_t)w0 * a.L, rows_total = (int64_t)a.T * a.L;
-                const int vk = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.skd.t * 2);
-                const int vv = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.svd.t * 2);
+                const int vk = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.skd.t * 2, a.D);
+                const int vv = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.svd.t * 2, a.Dv);
                 check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + anchor * a.skd.t,
                           nrows > 0 ? mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u) : 0u, vk, 0, 16, kt + i * 1024,
                           lds_bytes, vk == kPadOffset);
@@ -332,7 +332,7 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
                           lds_bytes, vv == kPadOffset);
                 continue;
               }
-              const int voffk = own.lane_offset(i, (int)a.skd.t * 2), voffv = own.lane_offset(i, (int)a.svd.t * 2);
+              const int voffk = own.lane_offset(i, (int)a.skd.t * 2, a.D), voffv = own.lane_offset(i, (int)a.svd.t * 2, a.Dv);
               check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + (int64_t)col0 * a.skd.t,
                         nrows > 0 ? (uint32_t)nrows * (uint32_t)a.skd.t * 2u : 0u, voffk, 0, 16, kt + i * 1024, lds_bytes,
                         voffk == kPadOffset);
@@ -363,7 +363,7 @@ void walk_delta(const KArgs& a_in) {
       const KArgs a = seq_args(a_in, b);
       const int r = rb * RPB + tid / TPR, c = (tid % TPR) * 8;
       ctx("delta_kernel", (int)block, tid >> 6, tid & 63, "o, do rows and the row sum");
-      if (r < a.Tq && c < a.D) {
+      if (r < a.Tq && c < a.Dv) {
         check_access("o", a.o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + c, 16, false);
         check_access("do", a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + c, 16, false);
       }
@@ -410,7 +410,7 @@ void walk_dkv(const KArgs& a_in) {
         const int64_t st = role_b ? (dep ? a.svd.t : a.sv.t) : (dep ? a.skd.t : a.sk.t);
         const char* sname = role_b ? (dep ? "vd" : "v") : (dep ? "kd" : "k");
         for (int ks = 0; ks < KS; ks++)
-          if (valid && 32 * ks + 8 * q4 < a.D) check_access(sname, src + crow * st + 32 * ks + 8 * q4, 16, false);
+          if (valid && 32 * ks + 8 * q4 < (role_b ? a.Dv : a.D)) check_access(sname, src + crow * st + 32 * ks + 8 * q4, 16, false);
         if (!valid) continue;
         ctx("dkv_kernel", (int)block, wave, lane, "gradient rows");
         if (nseg > 1 && !dep) {  // a row segment: fp32 partial sums, all HD columns of the tile width
@@ -426,13 +426,13 @@ void walk_dkv(const KArgs& a_in) {
                                  : (dep ? a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + crow * a.sdkd.t
                                         : a.dk + b * a.sdk.b + hkv * a.sdk.h + crow * a.sdk.t);
         for (int d = 0; d < MB; d++)
-          if (16 * d + 4 * q4 < a.D) check_access(oname, outp + 16 * d + 4 * q4, 8, true);
+          if (16 * d + 4 * q4 < (role_b ? a.D : a.Dv)) check_access(oname, outp + 16 * d + 4 * q4, 8, true);
       }
       // the streamed query tiles: per query head, from the top tile down, stages in turn
       Loader ld;
-      ld.init(tid, a.D);
+      ld.init(tid);
       const uint32_t q_row_bytes = (uint32_t)a.sq.t * 2u, do_row_bytes = (uint32_t)a.sdo.t * 2u;
-      const int voff_q = ld.lane_offset((int)q_row_bytes), voff_do = ld.lane_offset((int)do_row_bytes);
+      const int voff_q = ld.lane_offset((int)q_row_bytes, a.D), voff_do = ld.lane_offset((int)do_row_bytes, a.Dv);
       const int voff_stat = wave == 0 ? lane * a.Hq * 4 : lane * 4;
       const uint32_t stat_row_bytes = wave == 0 ? (uint32_t)a.Hq * 4u : 4u;
       int ld_st = 0;
@@ -449,9 +449,9 @@ void walk_dkv(const KArgs& a_in) {
           ctx("dkv_kernel", (int)block, wave, lane, "query tile (Q, dO)");
           for (int k = 0; k < Loader::N; k++) {
             check_dma("q", qp, rows * q_row_bytes, voff_q, k * 8 * Loader::RPW * (int)q_row_bytes, 16, lds_q + k * 8 * 1024,
-                      lds_bytes, ld.gchunk < 0);
+                      lds_bytes, ld.pads(a.D));
             check_dma("do", dop, rows * do_row_bytes, voff_do, k * 8 * Loader::RPW * (int)do_row_bytes, 16,
-                      lds_q + BM * HD * 2 + k * 8 * 1024, lds_bytes, ld.gchunk < 0);
+                      lds_q + BM * HD * 2 + k * 8 * 1024, lds_bytes, ld.pads(a.Dv));
           }
           if (wave < 2) {
             ctx("dkv_kernel", (int)block, wave, lane, wave == 0 ? "query tile lse" : "query tile row sums");
@@ -483,7 +483,7 @@ void walk_reduce(const KArgs& a) {
       for (int sg = 0; sg < a.dkv_split; sg++) check_access("part", src + sg * plane, 32, false);
       uint16_t* outp = which == 0 ? a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t
                                   : a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t;
-      if (8 * sub < a.D) check_access(which == 0 ? "dk" : "dv", outp + 8 * sub, 16, true);
+      if (8 * sub < (which == 0 ? a.D : a.Dv)) check_access(which == 0 ? "dk" : "dv", outp + 8 * sub, 16, true);
     }
   }
 }
@@ -509,15 +509,15 @@ void walk_chunk_depth(const KArgs& a_in) {
     for (int tid = 0; tid < 256; tid++) {
       const int lane = tid & 63, wave = tid >> 6;
       Loader ld;
-      ld.init(tid, a.D);
+      ld.init(tid);
       ctx("chunk_depth_kernel", (int)block, wave, lane, "the chunk's Q, dO, lse, row sums");
       for (int i = 0; i < Loader::N; i++) {
         check_dma("q", a.q + b * a.sq.b + hkv * a.sq.h + (int64_t)r0 * a.sq.t, Loader::anchored_bytes(a.sq.t, r0, r_end),
-                  ld.lane_offset((int)a.sq.t * 2), Loader::rows_before(i) * (int)a.sq.t * 2, 16, (uint32_t)ld.lds_elems(i) * 2,
-                  lds_bytes, ld.gchunk < 0);
+                  ld.lane_offset((int)a.sq.t * 2, a.D), Loader::rows_before(i) * (int)a.sq.t * 2, 16, (uint32_t)ld.lds_elems(i) * 2,
+                  lds_bytes, ld.pads(a.D));
         check_dma("do", a.d_o + b * a.sdo.b + hkv * a.sdo.h + (int64_t)r0 * a.sdo.t, Loader::anchored_bytes(a.sdo.t, r0, r_end),
-                  ld.lane_offset((int)a.sdo.t * 2), Loader::rows_before(i) * (int)a.sdo.t * 2, 16,
-                  (uint32_t)(BM * HD + ld.lds_elems(i)) * 2, lds_bytes, ld.gchunk < 0);
+                  ld.lane_offset((int)a.sdo.t * 2, a.Dv), Loader::rows_before(i) * (int)a.sdo.t * 2, 16,
+                  (uint32_t)(BM * HD + ld.lds_elems(i)) * 2, lds_bytes, ld.pads(a.Dv));
       }
       if (tid < BM && r0 + tid < r_end) {
         check_access("lse", a.lse + ((int64_t)b * a.Tq + r0 + tid) * a.Hq + hkv, 4, false);
@@ -526,34 +526,34 @@ void walk_chunk_depth(const KArgs& a_in) {
       const int prow = lane / CH, pch = lane % CH;
       const uint32_t wt = (uint32_t)(2 * BM * HD + wave * 32 * HD) * 2;
       WaveTileLoader<HD> own;
-      own.init(lane, a.D);
+      own.init(lane);
       for (int cb = t0 * a.Lv + wave * 32; cb < c_end; cb += 128) {
         const int nrows = imin(32, c_end - cb);
         for (int i = 0; i < NPASS; i++) {
           const int row = i * RPW + prow, lch = pch ^ Tile<HD>::swz(row);
-          const bool pad = !(lch * 8 < a.D);
+          const bool pad_k = !(lch * 8 < a.D), pad_v = !(lch * 8 < a.Dv);
           ctx("chunk_depth_kernel", (int)block, wave, lane, "depth K / V rows");
           if (a.Lv != a.L) {
             const int w0 = cb / a.Lv, l0 = cb - w0 * a.Lv;
             const int64_t anchor = (int64_t)w0 * a.L, rows_total = (int64_t)a.T * a.L;
-            const int vk = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.skd.t * 2);
-            const int vv = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.svd.t * 2);
+            const int vk = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.skd.t * 2, a.D);
+            const int vv = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.svd.t * 2, a.Dv);
             check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + anchor * a.skd.t,
                       mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u), vk, 0, 16, wt + i * 1024, lds_bytes, vk == kPadOffset);
             check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + anchor * a.svd.t,
                       mapped_bytes(anchor, rows_total, (uint32_t)a.svd.t * 2u), vv, 0, 16, wt + i * 1024, lds_bytes, vv == kPadOffset);
           } else {
-            const int vk = own.lane_offset(i, (int)a.skd.t * 2), vv = own.lane_offset(i, (int)a.svd.t * 2);
+            const int vk = own.lane_offset(i, (int)a.skd.t * 2, a.D), vv = own.lane_offset(i, (int)a.svd.t * 2, a.Dv);
             check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + (int64_t)cb * a.skd.t, (uint32_t)nrows * (uint32_t)a.skd.t * 2u,
-                      vk, 0, 16, wt + i * 1024, lds_bytes, pad);
+                      vk, 0, 16, wt + i * 1024, lds_bytes, pad_k);
             check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + (int64_t)cb * a.svd.t, (uint32_t)nrows * (uint32_t)a.svd.t * 2u,
-                      vv, 0, 16, wt + i * 1024, lds_bytes, pad);
+                      vv, 0, 16, wt + i * 1024, lds_bytes, pad_v);
           }
           ctx("chunk_depth_kernel", (int)block, wave, lane, "depth gradient rows");
-          if (cb + row < c_end && !pad) {
+          if (cb + row < c_end) {
             const int64_t prow_t = depth_row_of(a, cb + row);
-            check_access("dkd", a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + prow_t * a.sdkd.t + lch * 8, 16, true);
-            check_access("dvd", a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + prow_t * a.sdvd.t + lch * 8, 16, true);
+            if (!pad_k) check_access("dkd", a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + prow_t * a.sdkd.t + lch * 8, 16, true);
+            if (!pad_v) check_access("dvd", a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + prow_t * a.sdvd.t + lch * 8, 16, true);
           }
         }
       }
@@ -574,10 +574,10 @@ void walk_zero_unfilled(const KArgs& a) {
     const int h = (int)(rest % a.Hkv);
     rest /= a.Hkv;
     const int64_t row = rest % rows, b = rest / rows;
-    if (b >= batches || 8 * sub >= a.D || (int)(row % a.L) < a.Lv) continue;
+    if (b >= batches || (int)(row % a.L) < a.Lv) continue;
     ctx("zero_unfilled_slots_kernel", (int)(gid / 256), (int)(gid % 256) >> 6, (int)(gid & 63), "gradient rows of empty slots");
-    check_access("dkd", a.dkd + b * a.sdkd.b + h * a.sdkd.h + row * a.sdkd.t + 8 * sub, 16, true);
-    check_access("dvd", a.dvd + b * a.sdvd.b + h * a.sdvd.h + row * a.sdvd.t + 8 * sub, 16, true);
+    if (8 * sub < a.D) check_access("dkd", a.dkd + b * a.sdkd.b + h * a.sdkd.h + row * a.sdkd.t + 8 * sub, 16, true);
+    if (8 * sub < a.Dv) check_access("dvd", a.dvd + b * a.sdvd.b + h * a.sdvd.h + row * a.sdvd.t + 8 * sub, 16, true);
   }
 }
 
@@ -597,34 +597,28 @@ void walk_depth_cols(const KArgs& a_in) {
       const int64_t c = (int64_t)(block / BHk) * CPB + wave * CPW + lane / LPC;
       if (c >= (int64_t)a.T * a.L) continue;
       const int w = (int)(c / a.L), slot = (int)(c - (int64_t)w * a.L);
-      const bool in_dim = 8 * sub < a.D;
+      const bool in_k = 8 * sub < a.D, in_v = 8 * sub < a.Dv;
       ctx("depth_cols_kernel", (int)block, wave, lane, "depth column");
       uint16_t* dk_out = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + c * a.sdkd.t + 8 * sub;
       uint16_t* dv_out = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + c * a.sdvd.t + 8 * sub;
       if (slot >= a.Lv) {
-        if (!a.accum_depth && in_dim) {
-          check_access("dkd", dk_out, 16, true);
-          check_access("dvd", dv_out, 16, true);
+        if (!a.accum_depth) {
+          if (in_k) check_access("dkd", dk_out, 16, true);
+          if (in_v) check_access("dvd", dv_out, 16, true);
         }
         continue;
       }
-      if (in_dim) {
-        check_access("kd", a.kd + b * a.skd.b + hkv * a.skd.h + c * a.skd.t + 8 * sub, 16, false);
-        check_access("vd", a.vd + b * a.svd.b + hkv * a.svd.h + c * a.svd.t + 8 * sub, 16, false);
-      }
+      if (in_k) check_access("kd", a.kd + b * a.skd.b + hkv * a.skd.h + c * a.skd.t + 8 * sub, 16, false);
+      if (in_v) check_access("vd", a.vd + b * a.svd.b + hkv * a.svd.h + c * a.svd.t + 8 * sub, 16, false);
       for (int gq = 0; gq < a.Gf; gq++) {
         const int64_t r = (int64_t)w * a.Gf + gq;
-        if (in_dim) {
-          check_access("q", a.q + b * a.sq.b + hkv * a.sq.h + 8 * sub + r * a.sq.t, 16, false);
-          check_access("do", a.d_o + b * a.sdo.b + hkv * a.sdo.h + 8 * sub + r * a.sdo.t, 16, false);
-        }
+        if (in_k) check_access("q", a.q + b * a.sq.b + hkv * a.sq.h + 8 * sub + r * a.sq.t, 16, false);
+        if (in_v) check_access("do", a.d_o + b * a.sdo.b + hkv * a.sdo.h + 8 * sub + r * a.sdo.t, 16, false);
         check_access("lse", a.lse + ((int64_t)b * a.Tq + r) * a.Hq + hkv, 4, false);
         check_access("delta", a.delta + ((int64_t)b * a.Hq + hkv) * a.delta_pitch + r, 4, false);
       }
-      if (in_dim) {
-        check_access("dkd", dk_out, 16, true);
-        check_access("dvd", dv_out, 16, true);
-      }
+      if (in_k) check_access("dkd", dk_out, 16, true);
+      if (in_v) check_access("dvd", dv_out, 16, true);
     }
 }
 
@@ -706,14 +700,15 @@ void walk_all(const Case& c, const KArgs& a) {
 }  // namespace
 
 int main(int argc, char** argv) {
-  if (argc < 13) {
-    fprintf(stderr, "usage: %s HD D H G L Lv mode chunk_tokens split packed n len0 [len1 ...]\n", argv[0]);
+  if (argc < 14) {
+    fprintf(stderr, "usage: %s HD D Dv H G L Lv mode chunk_tokens split packed n len0 [len1 ...]\n", argv[0]);
     return 2;
   }
   Case c;
   int i = 1;
   c.HD = atoi(argv[i++]);
   c.D = atoi(argv[i++]);
+  c.Dv = atoi(argv[i++]);
   c.H = atoi(argv[i++]);
   c.G = atoi(argv[i++]);
   c.L = atoi(argv[i++]);

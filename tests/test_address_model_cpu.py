@@ -36,9 +36,10 @@ def tile_width(D):
     return 64 if D <= 64 else 128 if D <= 128 else 256
 
 
-def run(walker, lengths, H, D, L, G, mode, cb=0, packed=True, B=1, Lv=0, split=1, env=None):
+def run(walker, lengths, H, D, L, G, mode, cb=0, packed=True, B=1, Lv=0, split=1, env=None, Dv=None):
     n = len(lengths) if packed else B
-    args = [walker, tile_width(D), D, H, G, L, Lv, MODES[mode], cb, split, int(packed), n] + list(lengths)
+    Dv = D if Dv is None else Dv
+    args = [walker, tile_width(max(D, Dv)), D, Dv, H, G, L, Lv, MODES[mode], cb, split, int(packed), n] + list(lengths)
     e = dict(os.environ)
     e.update(env or {})
     r = subprocess.run([str(x) for x in args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=e,
@@ -120,6 +121,22 @@ def test_packed_batches(walker, case):
 def test_fixed_length_batches(walker, case):
     B, T, H, D, L, G, mode, cb, Lv = case
     rc, out = run(walker, (T,), H, D, L, G, mode, cb, packed=False, B=B, Lv=Lv)
+    assert rc == 0 and out.startswith("OK"), out
+
+
+@pytest.mark.parametrize("case", [
+    # B, T, H, D, Dv, L, G, mode, chunk tokens, Lv: value head dim different from the key head dim (one tile width)
+    (2, 150, 2, 64, 32, 5, 2, "causal", 0, 0),
+    (1, 197, 3, 64, 128, 4, 1, "noncausal", 0, 0),
+    (1, 300, 2, 128, 96, 6, 4, "chunk_visible", 16, 0),
+    (1, 260, 1, 40, 64, 3, 4, "chunk_visible", 40, 2),
+    (2, 60, 2, 128, 256, 3, 1, "depth_only", 0, 0),
+    (1, 333, 2, 192, 64, 0, 4, "plain", 0, 0),
+    (1, 2100, 1, 128, 64, 2, 2, "causal", 0, 1),
+], ids=lambda c: f"{c[7]}-D{c[3]}-Dv{c[4]}")
+def test_value_head_dim_differs(walker, case):
+    B, T, H, D, Dv, L, G, mode, cb, Lv = case
+    rc, out = run(walker, (T,), H, D, L, G, mode, cb, packed=False, B=B, Lv=Lv, Dv=Dv)
     assert rc == 0 and out.startswith("OK"), out
 
 

@@ -116,7 +116,8 @@ def test_matrix_core_routing_rule_is_the_librarys():
                         pb = ops.PackedBatch(cu, 2, 8, 13, host if packed == "with_host" else None)
                         if packed == "with_host":
                             d.cu_seqlens_host = ctypes.cast(host, ctypes.c_void_p)
-                    want = dtype != _lib.FP32 and D % 8 == 0 and Dv == D and not (D > 128 and packed == "device_only")
+                    want = (dtype != _lib.FP32 and D % 8 == 0 and Dv % 8 == 0
+                            and not (max(D, Dv) > 128 and packed == "device_only"))
                     assert lib.moda_hip_uses_matrix_cores(ctypes.byref(d)) == int(want), (dtype, D, Dv, packed)
                     q, v = torch.zeros(1, 8, 1, D, dtype=tdt), torch.zeros(1, 8, 1, Dv, dtype=tdt)
                     assert ops._matrix_core_path(q, v, pb) == want, (dtype, D, Dv, packed)

@@ -90,7 +90,15 @@ def check_l2(name, got, ref, dtype, what="", blocks=16):
             f"{what} {name}: rows [{a},{b}) relative L2 error {num / max(den, 1e-30):.3e} > {tol}"
 
 
-def compare_all(got, ref, dtype, what):
+def numerics(got, ref):
+    """max |err|, max |ref| and the relative L2 error of one tensor."""
+    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+    return (got - ref).abs().max().item(), ref.abs().max().item(), ((got - ref).norm() / ref.norm().clamp_min(1e-30)).item()
+
+
+def compare_all(got, ref, dtype, what, plain_atol=None):
+    """``plain_atol``: additionally hold every tensor but lse to max |err| <= plain_atol with no relative term (the
+    bar the benchmark configurations are quoted on) and print what was observed."""
     for n in ("o", "lse", "dq", "dk", "dv", "dkd", "dvd"):
         if ref[n] is None:
             assert got[n] is None, (what, n)
@@ -98,6 +106,10 @@ def compare_all(got, ref, dtype, what):
         check(n, got[n], ref[n], dtype, what)
         if n != "lse":
             check_l2(n, got[n], ref[n], dtype, what)
+        if plain_atol is not None:
+            err, mag, rel = numerics(got[n], ref[n])
+            say(f"NUMERICS {what} {n}: max_abs_err={err:.3e} max_abs_ref={mag:.3e} rel_l2={rel:.3e}")
+            assert err <= (LSE_ATOL if n == "lse" else plain_atol), f"{what} {n}: max |err| {err:.3e} > {plain_atol}"
 
 
 # ---------------------------------------------------------------------------
@@ -218,7 +230,7 @@ def test_config_c1_fp32(gpu_device):
     inp = oracle.make_inputs(1, 256, 4, 64, 4, 1, seed=0, dtype=torch.float32, prescale_q=True)
     ref = oracle.moda_dense_fwd_bwd(inp, 1.0, 1, "causal")
     got = run_hip(to_dev(inp, gpu_device), 1.0, 1, "causal")
-    compare_all(got, ref, torch.float32, "c1")
+    compare_all(got, ref, torch.float32, "c1", plain_atol=2e-4)
     # literal row loops on a slice of rows as a second opinion
     o_rows, lse_rows = oracle.moda_rows(inp["q"][:, :40], inp["k"][:, :40], inp["v"][:, :40], inp["kd"][:, :160],
                                         inp["vd"][:, :160], 1.0, 1, "causal")
@@ -250,7 +262,7 @@ def test_config_c2(gpu_device):
     got = run_hip(inp, sc, G, "causal")
     say("[c2] oracle")
     ref = _blockwise_on_gpu(inp, sc, G, "causal", 0, torch.bfloat16)
-    compare_all(got, ref, torch.bfloat16, "c2")
+    compare_all(got, ref, torch.bfloat16, "c2", plain_atol=2e-2)
     # row subsample against the dense form evaluated on the CPU
     rows = torch.tensor([0, 1, 5, 4095, 8191, 8192, 12345, 16383])
     cpu = {k: (None if v is None else v.cpu()) for k, v in inp.items()}
@@ -289,7 +301,7 @@ def test_config_c3_chunk_visible(gpu_device):
     torch.cuda.synchronize()
     say("[c3] oracle")
     ref = _blockwise_on_gpu(inp, sc, G, "chunk_visible", cb, torch.bfloat16)
-    compare_all(got, ref, torch.bfloat16, "c3")
+    compare_all(got, ref, torch.bfloat16, "c3", plain_atol=2e-2)
     _sum_invariants(inp, got, "c3")
     rows = torch.tensor([0, 63, 64, 65, 127, 32768, 65535], device=gpu_device)
     sub = oracle.moda_rows_subset(inp, rows, sc, G, "chunk_visible", cb)
@@ -312,7 +324,7 @@ def test_config_c4_headline_and_plain_twin(gpu_device):
     _sum_invariants(inp, got, "c4")
     say("[c4] oracle")
     ref = _blockwise_on_gpu(inp, sc, G, "causal", 0, torch.bfloat16, block_rows=8192)
-    compare_all(got, ref, torch.bfloat16, "c4")
+    compare_all(got, ref, torch.bfloat16, "c4", plain_atol=2e-2)
     del ref
     rows = torch.tensor([0, 3, 4, 131071, 131072, 262143], device=gpu_device)
     sub = oracle.moda_rows_subset(inp, rows, sc, G, "causal")
@@ -345,14 +357,14 @@ def test_config_c5_deit_noncausal_and_fda(gpu_device):
     sc = D ** -0.5
     got = run_hip(dev, sc, G, "noncausal")
     ref = oracle.moda_dense_fwd_bwd(inp, sc, G, "noncausal")
-    compare_all(got, ref, torch.bfloat16, "c5 noncausal")
+    compare_all(got, ref, torch.bfloat16, "c5 noncausal", plain_atol=2e-2)
     fda_in = dict(dev)
     fda_in["k"] = fda_in["v"] = None
     got = run_hip(fda_in, sc, G, "depth_only")
     cpu_in = dict(inp)
     cpu_in["k"] = cpu_in["v"] = None
     ref = oracle.moda_dense_fwd_bwd(cpu_in, sc, G, "depth_only")
-    compare_all(got, ref, torch.bfloat16, "c5 fda")
+    compare_all(got, ref, torch.bfloat16, "c5 fda", plain_atol=2e-2)
 
 
 # ---------------------------------------------------------------------------
@@ -844,6 +856,11 @@ def test_hip_graph_capture_and_replay(gpu_device):
     (1, 50, 2, 32, 96, 2, 1, "chunk_visible", 8, torch.float32),
     (1, 40, 2, 64, 32, 4, 2, "depth_only", 0, torch.bfloat16),
     (1, 33, 1, 96, 256, 0, 2, "causal", 0, torch.bfloat16),
+    (2, 300, 2, 128, 64, 6, 4, "chunk_visible", 16, torch.bfloat16),   # chunk kernel
+    (1, 260, 1, 40, 64, 3, 4, "chunk_visible", 40, torch.float16),     # depth column tiles, ring depth tiles
+    (1, 1024, 1, 128, 32, 2, 4, "causal", 0, torch.bfloat16),          # row segments + reduce
+    (3, 2100, 1, 64, 128, 2, 2, "causal", 0, torch.bfloat16),          # the throughput launch shape
+    (1, 200, 2, 72, 36, 3, 2, "causal", 0, torch.bfloat16),            # value head dim not a multiple of 8: vector-ALU kernels
 ], ids=lambda c: f"{c[7]}-D{c[3]}-Dv{c[4]}")
 def test_value_head_dim_differs_from_key_head_dim(gpu_device, case):
     import moda_amd
