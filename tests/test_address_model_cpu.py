@@ -93,6 +93,12 @@ FIXED = [
     (1, 100, 2, 256, 7, 4, "depth_only", 0, 0),
     (1, 1, 1, 256, 1, 1, "causal", 0, 0),
     (3, 2100, 1, 128, 2, 2, "causal", 0, 0),       # the throughput launch shape (256 rows per workgroup)
+    # query groups that fill a wave's 32 rows, or do not divide them (a token's rows then straddle waves and tiles)
+    (1, 77, 2, 128, 5, 8, "causal", 0, 0),
+    (1, 40, 1, 64, 3, 32, "noncausal", 0, 2),
+    (2, 90, 2, 128, 4, 3, "causal", 0, 0),
+    (1, 50, 1, 64, 6, 5, "depth_only", 0, 4),
+    (2, 1500, 1, 128, 3, 4, "causal", 0, 2),       # ... in the throughput launch shape, partially filled
     # what the per-sequence route launches for the packed case above: one fixed-length problem per sequence
     (1, 70, 1, 192, 5, 4, "chunk_visible", 8, 0),
     (1, 200, 1, 192, 5, 4, "chunk_visible", 8, 0),
