@@ -23,9 +23,6 @@
 // registers: every output row has one writer, no atomics, no partial buffers.
 #include <type_traits>
 
-// the tile loads of this file's kernels keep five wait states from vector-ALU writes of their scalar operands in
-// the compiled code (checked by tests/test_inline_asm_hazards_cpu.py): no padding inside the load blocks
-#define MODA_DMA_NOP 0
 #include "geometry.h"
 #include "kargs.h"
 #include "tile.h"
@@ -727,8 +724,9 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   if (in_v) *reinterpret_cast<i32x4*>(dv_out) = ov;
 }
 
-// Chunk-visible mode with a partially filled depth stream, not accumulating: the kernels above only visit the slots
-// that hold data, so the gradient rows of the other slots are written here (zeros).  One thread per 16 bytes of a
+// A partially filled depth stream, not accumulating: the chunk-visible kernels above, and the dQ kernel where it
+// forms the depth gradients itself, only visit the slots that hold data, so the gradient rows of the other slots
+// are written here (zeros).  One thread per 16 bytes of a
 // depth row; `rows`: depth rows per batch entry of the tensors (the whole packed axis for a packed batch).
 template <int HD>
 __global__ __launch_bounds__(256) void zero_unfilled_slots_kernel(const KArgs a, int64_t rows, int batches) {
@@ -798,7 +796,8 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
                  : allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_kernel<T, HD, false>), smem);
   if (ea != hipSuccess) return ea;
   // depth columns: vector kernel, except in chunk-visible mode where a column has up to G*Cb visible rows
-  const bool depth_by_columns = a.L > 0 && !a.chunk;
+  const bool in_dq = depth_grads_in_dq(a, HD);  // the dQ launch has formed the depth slots' dK and dV already
+  const bool depth_by_columns = a.L > 0 && !a.chunk && !in_dq;
   const int64_t n_seq_tiles = a.has_seq ? (a.T + BN - 1) / BN : 0;
   const bool depth_by_chunks = moda::depth_by_chunks(a, HD);
   const int64_t nblk = col_kernel_blocks(a, HD, BN, nseg);
@@ -819,7 +818,7 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
       if (er != hipSuccess) return er;
     }
   }
-  if (a.L > 0 && a.chunk && a.Lv != a.L && !a.accum_depth && (int64_t)a.B * a.T > 0) {
+  if (a.L > 0 && (a.chunk || in_dq) && a.Lv != a.L && !a.accum_depth && (int64_t)a.B * a.T > 0) {
     // packed batch: one row axis of all sequences (its length is the row-sum pitch / G), else B x T * L rows
     const int64_t rows = a.cu ? (int64_t)(a.delta_pitch / a.Gf) * a.L : (int64_t)a.T * a.L;
     const int batches = a.cu ? 1 : a.B;

@@ -121,10 +121,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   dep0 = __builtin_amdgcn_readfirstlane(dep0);
   const int ntiles = __builtin_amdgcn_readfirstlane(n_seq + n_dep);
 
-  // Wait states inside the tile-load blocks (see tile.h: lds_dma): the fixed-length instantiations with a fully
-  // filled depth stream (or none) keep their distance from vector-ALU scalar writes in the compiled code, the
-  // packed and partially filled ones do not (tests/test_inline_asm_hazards_cpu.py checks both)
-  constexpr int DMA_NOP = (VARLEN || PARTIAL) ? 3 : 0;
+  constexpr int DMA_NOP = MODA_DMA_NOP;
   typedef AsyncTileLoader<HD, BN, NT, DMA_NOP> Loader;
   constexpr int LPT = 2 * Loader::N;
   Loader ld;
@@ -251,7 +248,12 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     __syncthreads();
   }
 
-  if (own_depth) {
+  // Outside chunk-visible mode (when a token's rows never straddle waves) the pass over the wave's own depth
+  // columns also forms their dK and dV: see the second block below.
+  bool fused_depth = false;
+  constexpr bool FUSABLE = !NODEPTH && OWN_FITS && HD <= kDepthGradsInDqMaxWidth;
+  if constexpr (FUSABLE) fused_depth = depth_grads_in_dq(a, HD);
+  if (own_depth && !fused_depth) {
     // The wave's own depth columns, 32 at a time through a wave-private K tile and V tile cut out of the ring
     // (no workgroup barrier after the one that retires the ring).  The next V tile is fetched as soon as the
     // scores are out, the next K tile once dQ has its share.
@@ -294,6 +296,174 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     }
   }
 
+  // The wave's own depth columns when no other wave sees them (moda_v14.py:1251-1454, fda_v12.py:646-860 for
+  // their dK/dV): the products run the other way round here, S = Q Kd^T with the query rows on the accumulator
+  // registers (rows 4q + i of each 16-row block) and the depth column on the lane.  P and dS of the wave's 32 rows,
+  // rounded and packed, then ARE the operands (summation index = query row) of dVd^T = dO^T P and
+  // dKd^T = Q^T dS: one matrix instruction per 16 columns x 16 head-dim elements, nothing to accumulate across
+  // tiles.  Q^T and dO^T in that slot order are read once, through the private tiles before the first fetch.
+  // dQ needs dS with the columns as summation index: the rounded dS block crosses over through a small LDS block
+  // of the wave, which afterwards stages the gradient rows on their way out.
+  if constexpr (FUSABLE) {
+    if (fused_depth) {
+      static_assert(NB == 2, "the wave's 32 query rows are the 32 summation slots of one matrix instruction");
+      __syncthreads();
+      typedef WaveTileLoader<HD, DMA_NOP> Own;
+      const int wv = __builtin_amdgcn_readfirstlane(wave);
+      lds_ptr Kt = smem + wv * (2 * 32 * HD), Vt = Kt + 32 * HD;
+      lds_ptr stage = smem + Shape::W * 64 * HD + wv * (16 * HD);  // 16 rows of HD, or 32 x 32 for the dS block
+      const int rw0 = qt * BM + wv * WR;
+      if (rw0 < a.Tq) {
+        // Query row 16*nb + n goes to the tile row its lane reads as a row operand, slot_base(n >> 2) + (n & 3):
+        // the transposed read then delivers rows 4q + j and 16 + 4q + j as lane group q's eight summation slots,
+        // the order of the packed accumulators.
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+          for (int ks = 0; ks < KS; ks++) {
+            *reinterpret_cast<MODA_LDS i32x4*>(Kt + oa.row[ks] + 16 * nb * HD) = Qr[nb][ks];
+            *reinterpret_cast<MODA_LDS i32x4*>(Vt + oa.row[ks] + 16 * nb * HD) = dOr[nb][ks];
+          }
+        Own::reads_done();  // (the counter covers LDS writes as well)
+        i32x4 QT[MB], dOT[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+          QT[mb] = oa.tr_operand(Kt, 0, mb);
+          dOT[mb] = oa.tr_operand(Vt, 0, mb);
+        }
+        Own::reads_done();
+        // per accumulator register: base-2 LSE and minus delta of query row 16*nb + 4*q4 + i
+        f32x4 lse4[NB], del4[NB];
+        const int rq = rw0 + 4 * q4;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int r = rq + 16 * nb + i;
+            const bool ok = r < a.Tq;
+            lse4[nb][i] = ok ? a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq] : 0.f;
+            del4[nb][i] = ok ? a.delta[((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r] : 0.f;
+          }
+        const int gshift = __builtin_ctz(a.Gf);  // Gf divides 32: a power of two
+        const DepthSpan span = own_depth_span(a, rw0, WR);
+        const int c_beg = __builtin_amdgcn_readfirstlane(span.c_beg);
+        const int c_end = __builtin_amdgcn_readfirstlane(span.c_end);
+        const int nh = (c_end - c_beg + 31) / 32;
+        const uint16_t* kdp = a.kd + b * a.skd.b + hkv * a.skd.h;
+        const uint16_t* vdp = a.vd + b * a.svd.b + hkv * a.svd.h;
+        uint16_t* dkdp = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h;
+        uint16_t* dvdp = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h;
+        Own own;
+        own.init(lane);
+        auto fetch = [&](lds_ptr tile, const uint16_t* slice, int64_t stride, int col0, int d) {
+          const int nrows = min(32, c_end - col0);
+          if (PARTIAL)
+            own.fetch_mapped(tile, slice, stride, col0, nrows, (int64_t)a.T * a.L, a.L, a.Lv, d);
+          else
+            own.fetch(tile, slice, stride, col0, nrows, d);
+        };
+        const int lrow = slot_base(n >> 2) + (n & 3);  // tile row (of a 16-row block) whose column this lane holds
+        // 16 gradient rows (the columns cbase .. cbase + 15) leave through the staging block: the accumulators
+        // hold 8-byte pieces of 16 different rows per register, which the memory pipeline would take as 16 partial
+        // lines per store; written to LDS and read back by rows, every store covers whole rows.
+        constexpr int RPW = Own::RPW, NPASS = 16 / RPW;
+        auto stage_put = [&](int mb, const f32x4& x, float mul) {
+          i32x2 w;
+          w[0] = pack2<T>(x[0] * mul, x[1] * mul);
+          w[1] = pack2<T>(x[2] * mul, x[3] * mul);
+          *reinterpret_cast<MODA_LDS i32x2*>(stage + Tile<HD>::off(lrow, 2 * mb + (q4 >> 1)) + 4 * (q4 & 1)) = w;
+        };
+        auto flush = [&](uint16_t* base, int64_t stride, int cbase, int width) {
+          Own::reads_done();  // the block is written
+#pragma unroll
+          for (int i = 0; i < NPASS; i++) {
+            const int row = i * RPW + own.prow;
+            i32x4 val = *reinterpret_cast<MODA_LDS const i32x4*>(stage + i * 512 + lane * 8);
+            const int lch = own.pch ^ Tile<HD>::swz(row);
+            const int c = cbase + row;
+            if (c < c_end && lch * 8 < width) {
+              i32x4* dst = reinterpret_cast<i32x4*>(base + depth_row_of(a, c) * stride + lch * 8);
+              if (a.accum_depth) {  // add to what the row holds (this lane is the only writer of its 16 bytes)
+                const i32x4 old = *dst;
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                  float x0, x1, y0, y1;
+                  unpack2<T>(val[w], x0, x1);
+                  unpack2<T>(old[w], y0, y1);
+                  val[w] = pack2<T>(x0 + y0, x1 + y1);
+                }
+              }
+              *dst = val;
+            }
+          }
+          Own::reads_done();  // the block may be overwritten
+        };
+        fetch(Kt, kdp, a.skd.t, c_beg, a.D);
+        fetch(Vt, vdp, a.svd.t, c_beg, a.Dv);
+        MODA_LDS uint16_t* xs = (MODA_LDS uint16_t*)stage;  // dS block: [32 query rows][32 column slots]
+        for (int j = 0; j < nh; j++) {
+          const int col0 = c_beg + 32 * j;
+          const bool more = j + 1 < nh;
+          Own::template wait_but<0>();
+          f32x4 s[2][NB], dp[2][NB];
+          mfma16_rows2<T, HD, 2, NB, 2, true>(oa, Kt, Qr, s, Vt, dOr, dp, del4);
+          Own::reads_done();
+          if (more) fetch(Vt, vdp, a.svd.t, col0 + 32, a.Dv);  // K stays: dQ reads it transposed
+          i32x4 PA[2], DSA[2];
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++) {
+            const int c = col0 + 16 * cb + lrow;
+            const int tokc = c < c_end ? c / a.Lv : -2;
+            f32x4 p[NB], ds[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+              for (int i = 0; i < 4; i++) {
+                const int r = rq + 16 * nb + i;
+                float pv = fast_exp2(__builtin_fmaf(s[cb][nb][i], sc, -lse4[nb][i]));
+                pv = (r < a.Tq && (r >> gshift) == tokc) ? pv : 0.f;
+                p[nb][i] = pv;
+                ds[nb][i] = pv * dp[cb][nb][i];
+              }
+            PA[cb] = pack_slots<T>(p[0], p[1]);
+            DSA[cb] = pack_slots<T>(ds[0], ds[1]);
+            // the rounded dS block to LDS, a query row per 64-byte line, the column of tile row
+            // 16*cb + slot_base(g) + j in slot 8g + 4*cb + j: lane group g of the dQ product then reads its eight
+            // summation slots (tile rows slot_base(g) + j and 16 + slot_base(g) + j) as one 16-byte piece
+            const int slot = 8 * (n >> 2) + 4 * cb + (n & 3);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+              for (int i = 0; i < 4; i++) {
+                const int w = DSA[cb][2 * nb + (i >> 1)];
+                xs[(16 * nb + 4 * q4 + i) * 32 + slot] = (uint16_t)((i & 1) ? ((unsigned)w >> 16) : ((unsigned)w & 0xffffu));
+              }
+          }
+          Own::reads_done();
+          i32x4 DS[1][NB];
+#pragma unroll
+          for (int nb = 0; nb < NB; nb++) DS[0][nb] = *reinterpret_cast<MODA_LDS const i32x4*>(xs + (16 * nb + n) * 32 + 8 * q4);
+          TrPipe16<T, HD, 1, NB, 3> kt;
+          kt.prefetch(oa, Kt);
+          kt.run(oa, Kt, DS, dq);
+          Own::reads_done();
+          if (more) fetch(Kt, kdp, a.skd.t, col0 + 32, a.D);
+          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+            if (col0 + 16 * cb < c_end) {
+#pragma unroll
+              for (int mb = 0; mb < MB; mb++) stage_put(mb, mfma16<T>(dOT[mb], PA[cb], z), 1.f);
+              flush(dvdp, a.sdvd.t, col0 + 16 * cb, a.Dv);
+#pragma unroll
+              for (int mb = 0; mb < MB; mb++) stage_put(mb, mfma16<T>(QT[mb], DSA[cb], z), a.scale);
+              flush(dkdp, a.sdkd.t, col0 + 16 * cb, a.D);
+            }
+        }
+      }
+    }
+  }
+
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     const int r = qt * BM + wave * WR + 16 * nb + n;
@@ -323,8 +493,10 @@ hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
 template <typename T, int HD, typename Shape, int ADDR>
 hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
   // the ring, or one 32-column K tile and V tile per wave for the waves' own depth columns
-  constexpr size_t ring = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t), own = (size_t)Shape::W * 64 * HD * sizeof(uint16_t);
-  constexpr size_t smem = own <= 128 * 1024 ? std::max(ring, own) : ring;
+  // ... and, where the kernel forms the depth gradients, behind those a 16-row block per wave through which they leave
+  constexpr size_t ring = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t),
+                   own = (size_t)Shape::W * (64 + (HD <= kDepthGradsInDqMaxWidth ? 16 : 0)) * HD * sizeof(uint16_t);
+  constexpr size_t smem = (size_t)Shape::W * 64 * HD * sizeof(uint16_t) <= 128 * 1024 ? std::max(ring, own) : ring;
   static LdsAttrState attr;
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dq_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;

@@ -55,6 +55,18 @@ MODA_HD RowVis row_visibility(const KArgs& a, int r, int Ld) {
 // wave pair) are not streamed through the workgroup's ring: each wave fetches its own rows' span.
 MODA_HD bool waves_own_depth(const KArgs& a, int Ld) { return Ld > 0 && (!a.chunk || a.Cb * a.Gf <= 64); }
 
+// Outside chunk-visible mode a depth slot is seen by the Gf query rows of its own token only.  When those rows
+// always sit in one wave of the dQ kernel (32 rows per wave, Gf divides 32) the dQ kernel can form the slots' dK
+// and dV while their K and V rows are in its LDS tiles: no other wave contributes to them, and the depth stream is
+// read once per backward instead of twice.  Done for the 64-wide tiles only -- there the extra operands (Q^T and
+// dO^T of the wave's rows) fit the register file next to the dQ accumulators, and the shapes that use them are
+// bound by memory traffic; on the 128-wide tiles the same code spills and was measured slower than the separate
+// depth-column kernel, which every other case runs from the dK/dV launch.
+constexpr int kDepthGradsInDqMaxWidth = 64;
+MODA_HD bool depth_grads_in_dq(const KArgs& a, int HD) {
+  return a.L > 0 && !a.chunk && HD <= kDepthGradsInDqMaxWidth && 32 % a.Gf == 0;
+}
+
 // The column tiles of query tile qt: n_seq sequence tiles, of which the first n_full are seen completely by every
 // row of the workgroup, then n_dep depth tiles starting at flattened depth column dep0 (ring_depth: the depth
 // columns go through the ring at all).

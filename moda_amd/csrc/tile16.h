@@ -140,7 +140,9 @@ __device__ __forceinline__ void mfma16_rows(const Operand16<HD>& oa, lds_cptr ti
 
 // Two tiles against two register operand sets in one pipeline:
 // acc0[mb][nb] = rows(tile0) x breg0[nb], acc1[mb][nb] = init1[nb] + rows(tile1) x breg1[nb].
-template <typename T, int HD, int MBLK, int NB, int DEPTH, typename Hook = NoHook>
+// REG_A: the register operands go on the A side instead (the products come out transposed: lane n then holds the
+// tile row of its row operand, registers i the rows 4q + i of the register operand's block).
+template <typename T, int HD, int MBLK, int NB, int DEPTH, bool REG_A = false, typename Hook = NoHook>
 __device__ __forceinline__ void mfma16_rows2(const Operand16<HD>& oa, lds_cptr tile0,
                                              const i32x4 (&breg0)[NB][HD / 32], f32x4 (&acc0)[MBLK][NB],
                                              lds_cptr tile1, const i32x4 (&breg1)[NB][HD / 32],
@@ -163,9 +165,9 @@ __device__ __forceinline__ void mfma16_rows2(const Operand16<HD>& oa, lds_cptr t
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
       if (j & 1)
-        acc1[mb][nb] = mfma16<T>(ops[j], breg1[nb][ks], ks == 0 ? init1[nb] : acc1[mb][nb]);
+        acc1[mb][nb] = mfma16<T>(REG_A ? breg1[nb][ks] : ops[j], REG_A ? ops[j] : breg1[nb][ks], ks == 0 ? init1[nb] : acc1[mb][nb]);
       else
-        acc0[mb][nb] = mfma16<T>(ops[j], breg0[nb][ks], ks == 0 ? z : acc0[mb][nb]);
+        acc0[mb][nb] = mfma16<T>(REG_A ? breg0[nb][ks] : ops[j], REG_A ? ops[j] : breg0[nb][ks], ks == 0 ? z : acc0[mb][nb]);
     }
     __builtin_amdgcn_sched_barrier(0);
     hook(j);

@@ -341,6 +341,39 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
                         voffv == kPadOffset);
             }
           }
+          // dQ kernel outside chunk-visible mode: the same pass forms dK and dV of the wave's own depth columns.
+          // Lane (n, q4) reads the statistics of rows 16*nb + 4*q4 + i; the gradient rows leave 16 at a time
+          // through a staging block behind the private tiles, 16 bytes per lane (WaveTileLoader's row / chunk split).
+          if (dq && depth_grads_in_dq(a, HD)) {
+            if (rows_per_wave != 32) fail("%s: depth gradients need 32 rows per wave", kname);
+            const int q4 = lane >> 4;
+            const uint32_t stage = (uint32_t)Shape::W * 64 * HD * 2 + (uint32_t)wave * 16 * HD * 2;
+            if (stage + 16 * HD * 2 > lds_bytes) fail("%s: staging block past the LDS allocation", kname);
+            ctx(kname, (int)block, wave, lane, "own depth gradients");
+            for (int nb = 0; nb < 2; nb++)
+              for (int i = 0; i < 4; i++) {
+                const int r = rw0 + 16 * nb + 4 * q4 + i;
+                if (r >= a.Tq) continue;
+                check_access("lse", a.lse + ((int64_t)b * a.Tq + r) * a.Hq + hq, 4, false);
+                check_access("delta", a.delta + ((int64_t)b * a.Hq + hq) * (varlen ? a.delta_pitch : a.Tq) + r, 4, false);
+              }
+            constexpr int RPW = Own::RPW, NPASS = 16 / RPW;
+            for (int j = 0; j < nh; j++)
+              for (int cb = 0; cb < 2; cb++) {
+                const int cbase = span.c_beg + 32 * j + 16 * cb;
+                if (cbase >= span.c_end) continue;
+                for (int i = 0; i < NPASS; i++) {
+                  const int row = i * RPW + own.prow;
+                  const int lch = own.pch ^ Tile<HD>::swz(row);
+                  const int c = cbase + row;
+                  if (c >= span.c_end) continue;
+                  if (c / a.Lv >= a.T) fail("%s: depth column %d outside the stream", kname, c);
+                  const int64_t prow = depth_row_of(a, c);
+                  if (lch * 8 < a.Dv) check_access("dvd", a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + prow * a.sdvd.t + lch * 8, 16, true);
+                  if (lch * 8 < a.D) check_access("dkd", a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + prow * a.sdkd.t + lch * 8, 16, true);
+                }
+              }
+          }
         }
       }
     }
@@ -561,7 +594,8 @@ void walk_chunk_depth(const KArgs& a_in) {
   }
 }
 
-// the gradient rows of the slots without data (chunk-visible mode with a partially filled stream)
+// the gradient rows of the slots without data of a partially filled stream (launched where the kernels that form
+// the depth gradients only visit the slots that hold data)
 template <int HD>
 void walk_zero_unfilled(const KArgs& a) {
   constexpr int TPR = HD / 8;
@@ -660,8 +694,8 @@ void walk_all(const Case& c, const KArgs& a) {
   walk_delta<HD>(a);
   require_full("delta");
   auto ring_or_own = [&](int W, int NST) {
-    const uint32_t ring = (uint32_t)NST * 2 * 64 * HD * 2, own = (uint32_t)W * 64 * HD * 2;
-    return own <= 128 * 1024 ? std::max(ring, own) : ring;
+    const uint32_t ring = (uint32_t)NST * 2 * 64 * HD * 2, own = (uint32_t)W * (64 + (HD <= kDepthGradsInDqMaxWidth ? 16 : 0)) * HD * 2;
+    return (uint32_t)W * 64 * HD * 2 <= 128 * 1024 ? std::max(ring, own) : ring;
   };
   if constexpr (HD > 128) {
     walk_row_kernel<HD, RowWide, false>(a, true, 16, false, ring_or_own(RowWide::W, RowWide::NST), "dq_kernel(wide)");
@@ -682,12 +716,12 @@ void walk_all(const Case& c, const KArgs& a) {
     require_full("dv");
   }
   if (a.L > 0) {
-    if (a.chunk && a.Lv != a.L) walk_zero_unfilled<HD>(a);
+    if ((a.chunk || depth_grads_in_dq(a, HD)) && a.Lv != a.L) walk_zero_unfilled<HD>(a);
     if (a.chunk) {
       if constexpr (HD <= 128) {
         if (depth_by_chunks(a, HD)) walk_chunk_depth<HD>(a);
       }
-    } else {
+    } else if (!depth_grads_in_dq(a, HD)) {
       walk_depth_cols<HD>(a);
     }
     require_full("dkd");

@@ -181,6 +181,14 @@ VARIANTS = [
     (1, 197, 3, 160, 12, 1, "noncausal", 0, torch.bfloat16),
     (1, 100, 2, 256, 7, 4, "depth_only", 0, torch.float16),
     (1, 150, 1, 136, 2, 2, "causal", 0, torch.float16),
+    # 64-wide tiles outside chunk-visible mode: the dQ kernel forms the depth gradients when the query group divides
+    # a wave's 32 rows (groups of 8, 16, 32; the throughput launch shape), the depth-column kernel otherwise (3, 5)
+    (1, 77, 2, 64, 5, 8, "causal", 0, torch.bfloat16),
+    (1, 300, 1, 64, 2, 16, "depth_only", 0, torch.bfloat16),
+    (1, 40, 1, 64, 3, 32, "noncausal", 0, torch.float16),
+    (2, 90, 2, 64, 4, 3, "causal", 0, torch.bfloat16),
+    (1, 50, 1, 48, 6, 5, "depth_only", 0, torch.float16),
+    (8, 520, 8, 64, 1, 4, "causal", 0, torch.bfloat16),
 ]
 
 
