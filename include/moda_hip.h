@@ -173,12 +173,14 @@ int moda_hip_bwd(const moda_hip_desc* desc, const void* q, const void* k, const 
  * one stream (DQ and DKV read the workspace DELTA writes).  Lets a caller skip
  * dK/dV when only dQ is needed, or time the stages separately.  The reference
  * launches the same three steps one after another (moda_v14.py:1609, 1658,
- * 1698-1801).
+ * 1698-1801).  Which of DQ and DKV writes the depth gradients depends on the
+ * shape (outside chunk-visible mode the dQ kernel forms them itself for head
+ * dims up to 64 when G divides 32): dkd and dvd are complete once both have run.
  */
 enum moda_hip_bwd_stage {
   MODA_HIP_STAGE_DELTA = 1, /* row sums of o * do into the workspace  */
-  MODA_HIP_STAGE_DQ = 2,    /* dq                                     */
-  MODA_HIP_STAGE_DKV = 4,   /* dk, dv and, with a depth stream, dkd, dvd */
+  MODA_HIP_STAGE_DQ = 2,    /* dq (and, for some shapes, dkd and dvd: see below) */
+  MODA_HIP_STAGE_DKV = 4,   /* dk, dv and, with a depth stream, what is left of dkd, dvd */
   MODA_HIP_STAGE_ALL = 7
 };
 int moda_hip_bwd_stages(const moda_hip_desc* desc, const void* q, const void* k, const void* v,

@@ -292,10 +292,11 @@ inline hipError_t allow_dynamic_lds(LdsAttrState& state, const void* kernel, siz
 // spilled scalar) fewer than five wait states earlier sees the register's OLD value.  The compiler places
 // such writes right in front of the block when scalar registers are short (the forward kernels: dozens of sites),
 // so the block brings its own wait states: s_mov (1) + s_nop 3 (4), which also covers the one wait state m0 needs.
-// A kernel whose compiled code is known to keep its distance (tests/test_inline_asm_hazards_cpu.py checks every
-// tile load of every kernel in the compiler's output) may ask for NOP = 0 -- through the loaders' last template
-// argument, or for a whole source file by defining MODA_DMA_NOP as 0 before including this header -- and save the
-// four cycles per load; m0 still gets its one wait state.
+// NOP = 0 (the loaders' last template argument, or MODA_DMA_NOP defined as 0 before this header) leaves only the
+// one wait state m0 needs and is for experiments: whether the compiled code keeps its distance by itself changes
+// with unrelated edits (one more spilled scalar somewhere), so every kernel of the library keeps the wait states
+// -- about 0.3 % of the long-sequence step -- and tests/test_inline_asm_hazards_cpu.py checks every tile load of
+// every kernel in the compiler's output.
 #ifndef MODA_DMA_NOP
 #define MODA_DMA_NOP 3
 #endif
