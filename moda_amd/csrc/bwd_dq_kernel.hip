@@ -310,8 +310,11 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
       __syncthreads();
       typedef WaveTileLoader<HD, DMA_NOP> Own;
       const int wv = __builtin_amdgcn_readfirstlane(wave);
+      // two sets of a private K tile and V tile (the next tile's rows travel while this one is worked on), then
+      // the staging block: 16 rows of HD, or 32 x 32 for the dS block
       lds_ptr Kt = smem + wv * (2 * 32 * HD), Vt = Kt + 32 * HD;
-      lds_ptr stage = smem + Shape::W * 64 * HD + wv * (16 * HD);  // 16 rows of HD, or 32 x 32 for the dS block
+      constexpr int SET = Shape::W * 64 * HD;
+      lds_ptr stage = smem + 2 * SET + wv * (16 * HD);
       const int rw0 = qt * BM + wv * WR;
       if (rw0 < a.Tq) {
         // Query row 16*nb + n goes to the tile row its lane reads as a row operand, slot_base(n >> 2) + (n & 3):
@@ -401,15 +404,35 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
         fetch(Kt, kdp, a.skd.t, c_beg, a.D);
         fetch(Vt, vdp, a.svd.t, c_beg, a.Dv);
         MODA_LDS uint16_t* xs = (MODA_LDS uint16_t*)stage;  // dS block: [32 query rows][32 column slots]
+        // the gradient rows of one tile's columns from its packed P and dS
+        auto gradients = [&](const i32x4 (&PA)[2], const i32x4 (&DSA)[2], int col0) {
+          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+            if (col0 + 16 * cb < c_end) {
+#pragma unroll
+              for (int mb = 0; mb < MB; mb++) stage_put(mb, mfma16<T>(dOT[mb], PA[cb], z), 1.f);
+              flush(dvdp, a.sdvd.t, col0 + 16 * cb, a.Dv);
+#pragma unroll
+              for (int mb = 0; mb < MB; mb++) stage_put(mb, mfma16<T>(QT[mb], DSA[cb], z), a.scale);
+              flush(dkdp, a.sdkd.t, col0 + 16 * cb, a.D);
+            }
+        };
+        // Tile j: wait for its rows, send for tile j + 1 (other set), write out the gradient rows of tile j - 1, then
+        // scores, dS and dQ of tile j.  The stores of a tile are thus issued a whole tile before the next wait
+        // (the wave's memory counter covers loads and stores alike), the loads one tile ahead of their use.
+        i32x4 PA[2], DSA[2];
         for (int j = 0; j < nh; j++) {
           const int col0 = c_beg + 32 * j;
-          const bool more = j + 1 < nh;
+          lds_ptr Kc = Kt + (j & 1) * SET, Vc = Vt + (j & 1) * SET;
           Own::template wait_but<0>();
+          if (j + 1 < nh) {
+            fetch(Kt + ((j + 1) & 1) * SET, kdp, a.skd.t, col0 + 32, a.D);
+            fetch(Vt + ((j + 1) & 1) * SET, vdp, a.svd.t, col0 + 32, a.Dv);
+          }
+          if (j > 0) gradients(PA, DSA, col0 - 32);
           f32x4 s[2][NB], dp[2][NB];
-          mfma16_rows2<T, HD, 2, NB, 2, true>(oa, Kt, Qr, s, Vt, dOr, dp, del4);
-          Own::reads_done();
-          if (more) fetch(Vt, vdp, a.svd.t, col0 + 32, a.Dv);  // K stays: dQ reads it transposed
-          i32x4 PA[2], DSA[2];
+          mfma16_rows2<T, HD, 2, NB, 2, true>(oa, Kc, Qr, s, Vc, dOr, dp, del4);
 #pragma unroll
           for (int cb = 0; cb < 2; cb++) {
             const int c = col0 + 16 * cb + lrow;
@@ -444,22 +467,11 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
 #pragma unroll
           for (int nb = 0; nb < NB; nb++) DS[0][nb] = *reinterpret_cast<MODA_LDS const i32x4*>(xs + (16 * nb + n) * 32 + 8 * q4);
           TrPipe16<T, HD, 1, NB, 3> kt;
-          kt.prefetch(oa, Kt);
-          kt.run(oa, Kt, DS, dq);
-          Own::reads_done();
-          if (more) fetch(Kt, kdp, a.skd.t, col0 + 32, a.D);
-          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++)
-            if (col0 + 16 * cb < c_end) {
-#pragma unroll
-              for (int mb = 0; mb < MB; mb++) stage_put(mb, mfma16<T>(dOT[mb], PA[cb], z), 1.f);
-              flush(dvdp, a.sdvd.t, col0 + 16 * cb, a.Dv);
-#pragma unroll
-              for (int mb = 0; mb < MB; mb++) stage_put(mb, mfma16<T>(QT[mb], DSA[cb], z), a.scale);
-              flush(dkdp, a.sdkd.t, col0 + 16 * cb, a.D);
-            }
+          kt.prefetch(oa, Kc);
+          kt.run(oa, Kc, DS, dq);
+          Own::reads_done();  // this set and the staging block are free again
         }
+        if (nh > 0) gradients(PA, DSA, c_beg + 32 * (nh - 1));
       }
     }
   }
@@ -493,9 +505,10 @@ hipError_t launch_delta_t(const KArgs& a, hipStream_t stream) {
 template <typename T, int HD, typename Shape, int ADDR>
 hipError_t launch_dq_t_shape(const KArgs& a, hipStream_t stream) {
   // the ring, or one 32-column K tile and V tile per wave for the waves' own depth columns
-  // ... and, where the kernel forms the depth gradients, behind those a 16-row block per wave through which they leave
+  // ... and, where the kernel forms the depth gradients, a second set of those and a 16-row block per wave through
+  // which the gradients leave
   constexpr size_t ring = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t),
-                   own = (size_t)Shape::W * (64 + (HD <= kDepthGradsInDqMaxWidth ? 16 : 0)) * HD * sizeof(uint16_t);
+                   own = (size_t)Shape::W * (HD <= kDepthGradsInDqMaxWidth ? 2 * 64 + 16 : 64) * HD * sizeof(uint16_t);
   constexpr size_t smem = (size_t)Shape::W * 64 * HD * sizeof(uint16_t) <= 128 * 1024 ? std::max(ring, own) : ring;
   static LdsAttrState attr;
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dq_kernel<T, HD, Shape, ADDR>), smem);

@@ -347,7 +347,7 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
           if (dq && depth_grads_in_dq(a, HD)) {
             if (rows_per_wave != 32) fail("%s: depth gradients need 32 rows per wave", kname);
             const int q4 = lane >> 4;
-            const uint32_t stage = (uint32_t)Shape::W * 64 * HD * 2 + (uint32_t)wave * 16 * HD * 2;
+            const uint32_t stage = 2u * Shape::W * 64 * HD * 2 + (uint32_t)wave * 16 * HD * 2;
             if (stage + 16 * HD * 2 > lds_bytes) fail("%s: staging block past the LDS allocation", kname);
             ctx(kname, (int)block, wave, lane, "own depth gradients");
             for (int nb = 0; nb < 2; nb++)
@@ -694,7 +694,7 @@ void walk_all(const Case& c, const KArgs& a) {
   walk_delta<HD>(a);
   require_full("delta");
   auto ring_or_own = [&](int W, int NST) {
-    const uint32_t ring = (uint32_t)NST * 2 * 64 * HD * 2, own = (uint32_t)W * (64 + (HD <= kDepthGradsInDqMaxWidth ? 16 : 0)) * HD * 2;
+    const uint32_t ring = (uint32_t)NST * 2 * 64 * HD * 2, own = (uint32_t)W * (HD <= kDepthGradsInDqMaxWidth ? 2 * 64 + 16 : 64) * HD * 2;
     return (uint32_t)W * 64 * HD * 2 <= 128 * 1024 ? std::max(ring, own) : ring;
   };
   if constexpr (HD > 128) {
