@@ -178,7 +178,7 @@ int moda_hip_bwd(const moda_hip_desc* desc, const void* q, const void* k, const 
  * dims up to 64 when G divides 32): dkd and dvd are complete once both have run.
  */
 enum moda_hip_bwd_stage {
-  MODA_HIP_STAGE_DELTA = 1, /* row sums of o * do into the workspace  */
+  MODA_HIP_STAGE_DELTA = 1, /* row sums of o * do into the workspace (asked for together with DQ, the dQ kernel forms them) */
   MODA_HIP_STAGE_DQ = 2,    /* dq (and, for some shapes, dkd and dvd: see below) */
   MODA_HIP_STAGE_DKV = 4,   /* dk, dv and, with a depth stream, what is left of dkd, dvd */
   MODA_HIP_STAGE_ALL = 7

@@ -95,9 +95,31 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     }
     lse[nb] = 0.f;
     delta[nb] = 0.f;
-    if (valid) {
-      lse[nb] = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq];
-      delta[nb] = a.delta[((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r];
+    if (valid) lse[nb] = a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq];
+    float* drow = a.delta + ((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r;
+    if (a.own_delta) {
+      // minus rowsum(o * do) (moda_v14.py:525-539) from the dO pieces this lane holds anyway and the same pieces of
+      // o; the four lanes of a row add their shares and the first one leaves the sum for the kernels that follow
+      const uint16_t* orow = a.o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + 8 * q4;
+      float acc = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        i32x4 z = {0, 0, 0, 0};
+        const i32x4 ov = (valid && 32 * ks + 8 * q4 < a.Dv) ? *reinterpret_cast<const i32x4*>(orow + 32 * ks) : z;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+          float x0, x1, y0, y1;
+          unpack2<T>(ov[w], x0, x1);
+          unpack2<T>(dOr[nb][ks][w], y0, y1);
+          acc = __builtin_fmaf(x0, y0, acc);
+          acc = __builtin_fmaf(x1, y1, acc);
+        }
+      }
+      acc = quad_sum(acc);
+      delta[nb] = valid ? -acc : 0.f;
+      if (valid && q4 == 0) *drow = -acc;
+    } else if (valid) {
+      delta[nb] = *drow;
     }
     const RowVis vis = row_visibility(a, r, Ld);
     shi[nb] = vis.shi;
@@ -335,17 +357,16 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
           dOT[mb] = oa.tr_operand(Vt, 0, mb);
         }
         Own::reads_done();
-        // per accumulator register: base-2 LSE and minus delta of query row 16*nb + 4*q4 + i
+        // per accumulator register: base-2 LSE and minus delta of query row 16*nb + 4*q4 + i, from the lanes that
+        // hold those rows (lane n of the first sixteen holds row 16*nb + n; rows past the end carry zeros)
         f32x4 lse4[NB], del4[NB];
         const int rq = rw0 + 4 * q4;
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            const int r = rq + 16 * nb + i;
-            const bool ok = r < a.Tq;
-            lse4[nb][i] = ok ? a.lse[((int64_t)b * a.Tq + r) * a.Hq + hq] : 0.f;
-            del4[nb][i] = ok ? a.delta[((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + r] : 0.f;
+            lse4[nb][i] = __shfl(lse[nb], 4 * q4 + i, 64);
+            del4[nb][i] = __shfl(delta[nb], 4 * q4 + i, 64);
           }
         const int gshift = __builtin_ctz(a.Gf);  // Gf divides 32: a power of two
         const DepthSpan span = own_depth_span(a, rw0, WR);

@@ -416,7 +416,9 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = hipSuccess;
   if (use_mfma(d)) {
-    if (stages & MODA_HIP_STAGE_DELTA) e = moda::launch_delta(a, d->dtype, tile_width(d), s);
+    // with both stages asked for, the dQ kernel forms the row sums itself (one launch and one pass over o, do less)
+    a.own_delta = (stages & MODA_HIP_STAGE_DELTA) && (stages & MODA_HIP_STAGE_DQ) ? 1 : 0;
+    if ((stages & MODA_HIP_STAGE_DELTA) && !a.own_delta) e = moda::launch_delta(a, d->dtype, tile_width(d), s);
     if (e == hipSuccess && (stages & MODA_HIP_STAGE_DQ)) e = moda::launch_dq(a, d->dtype, tile_width(d), s);
     if (e == hipSuccess && (stages & MODA_HIP_STAGE_DKV)) e = moda::launch_dkv(a, d->dtype, tile_width(d), s);
   } else {

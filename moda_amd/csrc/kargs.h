@@ -27,6 +27,7 @@ struct KArgs {
   int Cb;    // chunk-visible: tokens per chunk
   int has_seq, causal, chunk;
   int accum_depth;  // dkd, dvd += (slots l >= Lv untouched) instead of = (slots l >= Lv zeroed)
+  int own_delta;    // the dQ kernel forms the row sums of o * do itself and leaves them in `delta` for the later kernels
   // Sequence dK/dV of launches too small to fill the device: the query rows of every column tile are cut into
   // `dkv_split` segments, one workgroup each, which leave fp32 partial sums in `dkv_part`
   // ([2 (dk, dv)][dkv_split][B][Hkv][T][D]); a second kernel adds them in segment order.  1 = no split.

@@ -158,6 +158,7 @@ KArgs make_args(const Case& c) {
   a.compute_units = 256;
   const int64_t qrows = plain ? T : (int64_t)T * c.G;
   a.delta_pitch = c.packed ? (int)qrows : a.Tq;
+  a.own_delta = 1;  // a whole backward: the dQ kernel forms the row sums (the delta kernel is walked as well)
   auto strides = [&](int64_t rows, int heads, int dim) { return Str3{rows * heads * dim, (int64_t)heads * dim, (int64_t)dim}; };
   // bytes of a dense [Bt, rows, heads, dim] tensor of 16-bit elements
   auto bytes = [&](int64_t rows, int heads, int dim) { return (uint64_t)Bt * rows * heads * dim * 2; };
@@ -239,12 +240,15 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
         for (int e = piece; e < HD; e += step) {
           if (e < a.D) check_access("q", a.q + b * a.sq.b + hq * a.sq.h + (int64_t)r * a.sq.t + e, 16, false);
           if (dq && e < a.Dv) check_access("do", a.d_o + b * a.sdo.b + hq * a.sdo.h + (int64_t)r * a.sdo.t + e, 16, false);
+          if (dq && a.own_delta && e < a.Dv) check_access("o", a.o + b * a.so.b + hq * a.so.h + (int64_t)r * a.so.t + e, 16, false);
         }
         const bool stat_lane = rows_per_wave == 32 ? (lane >> 5) == 0 : (lane >> 4) == 0;
         ctx(kname, (int)block, wave, lane, "row statistics and result rows");
         if (dq) {
           check_access("lse", a.lse + ((int64_t)b * a.Tq + r) * a.Hq + hq, 4, false);
-          check_access("delta", a.delta + ((int64_t)b * a.Hq + hq) * (varlen ? a.delta_pitch : a.Tq) + r, 4, false);
+          // the row sum: read, or formed here and left for the later kernels by the first of the row's four lanes
+          if (!a.own_delta || stat_lane)
+            check_access("delta", a.delta + ((int64_t)b * a.Hq + hq) * (varlen ? a.delta_pitch : a.Tq) + r, 4, a.own_delta != 0);
         } else if (stat_lane) {
           check_access("lse", a.lse + ((int64_t)b * a.Tq + r) * a.Hq + hq, 4, true);
         }
@@ -342,21 +346,13 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
             }
           }
           // dQ kernel outside chunk-visible mode: the same pass forms dK and dV of the wave's own depth columns.
-          // Lane (n, q4) reads the statistics of rows 16*nb + 4*q4 + i; the gradient rows leave 16 at a time
-          // through a staging block behind the private tiles, 16 bytes per lane (WaveTileLoader's row / chunk split).
+          // The gradient rows leave 16 at a time through a staging block behind the private tiles, 16 bytes per lane
+          // (WaveTileLoader's row / chunk split).
           if (dq && depth_grads_in_dq(a, HD)) {
             if (rows_per_wave != 32) fail("%s: depth gradients need 32 rows per wave", kname);
-            const int q4 = lane >> 4;
             const uint32_t stage = 2u * Shape::W * 64 * HD * 2 + (uint32_t)wave * 16 * HD * 2;
             if (stage + 16 * HD * 2 > lds_bytes) fail("%s: staging block past the LDS allocation", kname);
             ctx(kname, (int)block, wave, lane, "own depth gradients");
-            for (int nb = 0; nb < 2; nb++)
-              for (int i = 0; i < 4; i++) {
-                const int r = rw0 + 16 * nb + 4 * q4 + i;
-                if (r >= a.Tq) continue;
-                check_access("lse", a.lse + ((int64_t)b * a.Tq + r) * a.Hq + hq, 4, false);
-                check_access("delta", a.delta + ((int64_t)b * a.Hq + hq) * (varlen ? a.delta_pitch : a.Tq) + r, 4, false);
-              }
             constexpr int RPW = Own::RPW, NPASS = 16 / RPW;
             for (int j = 0; j < nh; j++)
               for (int cb = 0; cb < 2; cb++) {
@@ -691,8 +687,10 @@ void walk_all(const Case& c, const KArgs& a) {
   require_full("o");
   require_full("lse");
   // ---- backward
+  // the row sums: by the delta kernel when that stage is run alone, else inside the dQ kernel
   walk_delta<HD>(a);
   require_full("delta");
+  reset_writes("delta");
   auto ring_or_own = [&](int W, int NST) {
     const uint32_t ring = (uint32_t)NST * 2 * 64 * HD * 2, own = (uint32_t)W * (HD <= kDepthGradsInDqMaxWidth ? 2 * 64 + 16 : 64) * HD * 2;
     return (uint32_t)W * 64 * HD * 2 <= 128 * 1024 ? std::max(ring, own) : ring;
@@ -706,6 +704,7 @@ void walk_all(const Case& c, const KArgs& a) {
       walk_row_kernel<HD, RowLarge, false>(a, true, 32, true, ring_or_own(RowLarge::W, RowLarge::NST), "dq_kernel");
   }
   require_full("dq");
+  require_full("delta");
   walk_dkv<HD>(a);
   if (a.dkv_split > 1 && a.has_seq) {
     require_full("part");
