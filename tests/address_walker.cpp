@@ -322,6 +322,8 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
           for (int j = 0; j < nh; j++) {
             const int col0 = span.c_beg + 32 * j;
             const int nrows = imin(32, span.c_end - col0);
+            // where the dQ kernel forms the depth gradients it alternates between two sets of private tiles
+            const uint32_t set = (dq && depth_grads_in_dq(a, HD)) ? (uint32_t)(j & 1) * Shape::W * 64 * HD * 2 : 0u;
             for (int i = 0; i < Own::N; i++) {
               if (a.Lv != a.L) {
                 const int w0 = col0 / a.Lv, l0 = col0 - w0 * a.Lv;
@@ -329,19 +331,19 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
                 const int vk = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.skd.t * 2, a.D);
                 const int vv = own.mapped_offset(i, l0, a.L, a.Lv, nrows, (int)a.svd.t * 2, a.Dv);
                 check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + anchor * a.skd.t,
-                          nrows > 0 ? mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u) : 0u, vk, 0, 16, kt + i * 1024,
+                          nrows > 0 ? mapped_bytes(anchor, rows_total, (uint32_t)a.skd.t * 2u) : 0u, vk, 0, 16, kt + set + i * 1024,
                           lds_bytes, vk == kPadOffset);
                 check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + anchor * a.svd.t,
-                          nrows > 0 ? mapped_bytes(anchor, rows_total, (uint32_t)a.svd.t * 2u) : 0u, vv, 0, 16, vt + i * 1024,
+                          nrows > 0 ? mapped_bytes(anchor, rows_total, (uint32_t)a.svd.t * 2u) : 0u, vv, 0, 16, vt + set + i * 1024,
                           lds_bytes, vv == kPadOffset);
                 continue;
               }
               const int voffk = own.lane_offset(i, (int)a.skd.t * 2, a.D), voffv = own.lane_offset(i, (int)a.svd.t * 2, a.Dv);
               check_dma("kd", a.kd + b * a.skd.b + hkv * a.skd.h + (int64_t)col0 * a.skd.t,
-                        nrows > 0 ? (uint32_t)nrows * (uint32_t)a.skd.t * 2u : 0u, voffk, 0, 16, kt + i * 1024, lds_bytes,
+                        nrows > 0 ? (uint32_t)nrows * (uint32_t)a.skd.t * 2u : 0u, voffk, 0, 16, kt + set + i * 1024, lds_bytes,
                         voffk == kPadOffset);
               check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + (int64_t)col0 * a.svd.t,
-                        nrows > 0 ? (uint32_t)nrows * (uint32_t)a.svd.t * 2u : 0u, voffv, 0, 16, vt + i * 1024, lds_bytes,
+                        nrows > 0 ? (uint32_t)nrows * (uint32_t)a.svd.t * 2u : 0u, voffv, 0, 16, vt + set + i * 1024, lds_bytes,
                         voffv == kPadOffset);
             }
           }
