@@ -23,6 +23,7 @@ from .ops import (  # noqa: F401
     ParallelAttentionFunction,
     fold_gqa_heads,
     unfold_gqa_heads,
+    set_fp32_compute,
 )
 from .depth_cache import build_depth_cache, stack_depth, DepthCache  # noqa: F401
 from .modules import DepthStream, MoDAAttention, MoDAStack  # noqa: F401
@@ -42,6 +43,7 @@ __all__ = [
     "parallel_attn_bwd",
     "fold_gqa_heads",
     "unfold_gqa_heads",
+    "set_fp32_compute",
     "build_depth_cache",
     "stack_depth",
     "DepthCache",

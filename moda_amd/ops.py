@@ -27,6 +27,30 @@ from ._lib import Desc, Strides
 
 _DTYPES = {torch.bfloat16: _lib.BF16, torch.float16: _lib.FP16, torch.float32: _lib.FP32}
 
+# How fp32 tensors are computed.  "fp32": in fp32 on the vector-ALU kernels (exact to fp32 rounding, two orders of
+# magnitude slower than the matrix kernels).  "fp16" / "bf16": the inputs are rounded to that type, the matrix
+# kernels run, the results are widened again.  "fp16" is what the reference's own fp32 path amounts to: its
+# tl.dot calls (moda_v14.py:188, 209, 699-712) take the default input precision, which rounds fp32 operands to a
+# 10-bit mantissa (TF32) and accumulates in fp32 -- fp16 has the same mantissa; its range (6e-8 .. 65504) is the
+# caller's responsibility, "bf16" trades three mantissa bits for the fp32 range.
+_FP32_COMPUTE = "fp32"
+_FP32_COMPUTE_TYPES = {"fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+def set_fp32_compute(mode: str) -> str:
+    """Choose how fp32 tensors are computed ("fp32", "fp16" or "bf16", see above); returns the previous setting."""
+    global _FP32_COMPUTE
+    assert mode in ("fp32", "fp16", "bf16"), f"unknown fp32 compute mode {mode!r}"
+    previous, _FP32_COMPUTE = _FP32_COMPUTE, mode
+    return previous
+
+
+def _narrowed(*xs):
+    """fp32 tensors -> the 16-bit compute type chosen with set_fp32_compute (None stays None)."""
+    t = _FP32_COMPUTE_TYPES[_FP32_COMPUTE]
+    return tuple(None if x is None else x.to(t) for x in xs)
+
+
 # Query rows per chunk of the chunk-visible variant when the caller does not
 # say: the value the reference hard-wires in its launchers (moda_v16.py:581-585).
 DEFAULT_CHUNK_ROWS = 64
@@ -233,6 +257,9 @@ def _check_shapes(mode, q, k, v, kd, vd, G, o=None, do=None, lse=None):
 
 def _raw_fwd(mode, q, k, v, kd, vd, scale, G, chunk_tokens=0, depth_valid=None, packed=None):
     """Launch the forward kernels. Returns (o, lse)."""
+    if q.dtype == torch.float32 and _FP32_COMPUTE != "fp32":
+        o, lse = _raw_fwd(mode, *_narrowed(q, k, v, kd, vd), scale, G, chunk_tokens, depth_valid, packed)
+        return o.float(), lse
     _check_shapes(mode, q, k, v, kd, vd, G)
     _check_device(q)
     _same_dtype(q, k, v, kd, vd)
@@ -266,6 +293,17 @@ def _raw_bwd(mode, q, k, v, kd, vd, o, lse, do, scale, G, chunk_tokens=0, stages
     ``>= depth_valid`` untouched) instead of overwriting them."""
     assert not accumulate_depth or (out is not None and out[3] is not None and out[4] is not None), \
         "accumulate_depth needs the gradient buffers to add to"
+    if q.dtype == torch.float32 and _FP32_COMPUTE != "fp32":
+        # 16-bit gradients from the matrix kernels (without the accumulate flag: the slots without data come back
+        # as zeros), widened into the caller's fp32 buffers or added to them
+        got = _raw_bwd(mode, *_narrowed(q, k, v, kd, vd, o), lse, *_narrowed(do), scale, G, chunk_tokens, stages,
+                       None, None, depth_valid, packed, False)
+        if out is None:
+            return tuple(None if g_ is None else g_.float() for g_ in got)
+        for i, (dst, g_) in enumerate(zip(out, got)):
+            if dst is not None:
+                dst.add_(g_) if (accumulate_depth and i >= 3) else dst.copy_(g_)
+        return tuple(out)
     _check_shapes(mode, q, k, v, kd, vd, G, o=o, do=do, lse=lse)
     _check_device(q)
     _same_dtype(q, k, v, kd, vd, o, do)

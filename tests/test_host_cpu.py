@@ -388,3 +388,13 @@ def test_attention_module_mirrors_reference_parameters():
     assert s.context() == (None, None, None) and len(s) == 0
     with pytest.raises(RuntimeError, match="no CPU path"):
         m(torch.zeros(1, 8, 384))
+
+
+def test_fp32_compute_setting():
+    import moda_amd
+
+    assert moda_amd.set_fp32_compute("fp16") == "fp32"
+    assert moda_amd.set_fp32_compute("fp32") == "fp16"
+    with pytest.raises(AssertionError):
+        moda_amd.set_fp32_compute("tf32")
+    assert moda_amd.set_fp32_compute("fp32") == "fp32"

@@ -203,6 +203,47 @@ def test_variants(gpu_device, case):
     compare_all(got, ref, dtype, str(case))
 
 
+@pytest.mark.parametrize("case", [
+    # (B, T, H, D, L, G, mode, chunk tokens, compute type)
+    (1, 256, 4, 64, 4, 2, "causal", 0, "fp16"),          # the fp32 plumbing configuration of the benchmark list
+    (2, 197, 3, 64, 12, 1, "noncausal", 0, "fp16"),
+    (1, 300, 2, 128, 6, 4, "chunk_visible", 16, "bf16"),
+    (1, 100, 2, 96, 3, 2, "depth_only", 0, "fp16"),
+])
+def test_fp32_inputs_through_the_matrix_kernels(gpu_device, case):
+    """``set_fp32_compute("fp16" | "bf16")``: fp32 tensors are rounded to the 16-bit type, run on the matrix kernels and
+    come back as fp32 -- for fp16 the same operand precision as the reference's fp32 path (tl.dot's default input
+    precision keeps a 10-bit mantissa, moda_v14.py:188, 209).  Checked against the oracle on the UNROUNDED fp32 inputs
+    at the 16-bit type's tolerance; the default setting stays exact fp32 (every other fp32 case of this file)."""
+    import moda_amd
+    from moda_amd import ops
+
+    B, T, H, D, L, G, mode, cb, how = case
+    say(f"CASE fp32-compute {case}")
+    inp = oracle.make_inputs(B, T, H, D, L, G, seed=41, dtype=torch.float32, std=0.5, depth_only=(mode == "depth_only"))
+    sc = D ** -0.5
+    ref = oracle.moda_dense_fwd_bwd(inp, sc, G, mode, cb)
+    previous = moda_amd.set_fp32_compute(how)
+    try:
+        assert previous == "fp32"
+        got = run_hip(to_dev(inp, gpu_device), sc, G, mode, cb)
+        # accumulate flag: fp32 buffers that already hold something
+        dev = to_dev(inp, gpu_device)
+        m = MODE_ID[mode]
+        o, lse = ops._raw_fwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], sc, G, cb)
+        held = tuple(None if dev[n] is None else torch.ones_like(dev[n]) for n in ("q", "k", "v", "kd", "vd"))
+        ops._raw_bwd(m, dev["q"], dev["k"], dev["v"], dev["kd"], dev["vd"], o, lse, dev["do"], sc, G, cb, out=held,
+                     accumulate_depth=True)
+    finally:
+        assert moda_amd.set_fp32_compute(previous) == how
+    narrow = torch.float16 if how == "fp16" else torch.bfloat16
+    for name, x in got.items():
+        assert x is None or x.dtype == torch.float32, name
+    compare_all(got, ref, narrow, f"fp32 via {how} {case}")
+    assert torch.equal(held[0], got["dq"]) and (held[1] is None or torch.equal(held[1], got["dk"]))
+    assert torch.equal(held[3], got["dkd"] + 1.0) and torch.equal(held[4], got["dvd"] + 1.0)
+
+
 def test_golden_fixture(gpu_device):
     """Committed fixture (tests/golden/moda_small.npz) against the HIP kernels in fp32 and bf16."""
     import os
