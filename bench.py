@@ -276,7 +276,19 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # kernel of the same runs): FETCH_SIZE counts half of the bytes read, WRITE_SIZE all bytes written
 PMC_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
 KERNEL_NAMES = ("fwd_kernel", "fwd_wide_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "dkv_reduce_kernel", "depth_cols_kernel",
-                "chunk_depth_kernel", "reorg_kernel")
+                "depth_token_handed_kernel", "depth_cols_handed_kernel", "chunk_depth_kernel", "reorg_kernel")
+
+
+def depth_gradient_kernel(mode, D, G):
+    """Name of the launch that forms dkd, dvd after dkv_kernel (moda_amd/csrc/geometry.h: depth_grads_in_dq,
+    depth_scores_from_dq), or None where the dQ kernel forms them itself."""
+    if mode == "chunk_visible":
+        return "chunk_depth_kernel"
+    if D <= 64 and 32 % G == 0:
+        return None
+    if D <= 128:
+        return "depth_token_handed_kernel" if G <= 4 else "depth_cols_handed_kernel"
+    return "depth_cols_kernel"
 
 
 def recorded_traffic(workload):
@@ -470,16 +482,15 @@ def main():
     }
     dom = max(("fwd_kernel", "dq_kernel", "dkv_kernel"), key=lambda n: kernels[n]["ms"])
     traffic = recorded_traffic(args.workload) or {}
-    # the dK/dV stage is timed as a whole: outside chunk-visible mode it is dkv_kernel followed by the HBM-bound
-    # depth_cols_kernel
-    # (chunk-visible: dkv_kernel followed by chunk_depth_kernel; light launches add dkv_reduce_kernel)
-    two_launches = dom == "dkv_kernel" and L > 0
-    depth_kernel = "chunk_depth_kernel" if mode == "chunk_visible" else "depth_cols_kernel"
+    # the dK/dV stage is timed as a whole: dkv_kernel followed by the HBM-bound launch that forms the depth gradients
+    # (where the dQ kernel does not form them itself; light launches add dkv_reduce_kernel)
+    depth_kernel = depth_gradient_kernel(mode, D, G) if L > 0 else None
+    two_launches = dom == "dkv_kernel" and depth_kernel is not None
     dom_traffic = None
     if dom in traffic:
         dom_traffic = traffic[dom]["bytes"]
         if dom == "dkv_kernel":
-            dom_traffic += sum(traffic.get(k, {}).get("bytes", 0.0) for k in (depth_kernel, "dkv_reduce_kernel"))
+            dom_traffic += sum(traffic.get(k, {}).get("bytes", 0.0) for k in (depth_kernel, "dkv_reduce_kernel") if k)
     roofline = {
         "bound": "mfma",
         "kernel": f"dkv_kernel + {depth_kernel}" if two_launches else dom,
@@ -495,7 +506,8 @@ def main():
         mb = min_hbm_bytes(B, T, Hkv, G, D, L, mode)
         gbs = mb / (r["ms_step"] * 1e-3) / 1e9
         whole = sum(v["bytes"] for k, v in traffic.items() if k != "reorg_kernel") if traffic else None
-        roofline = {"bound": "hbm", "kernel": "fwd_kernel + delta_kernel + dq_kernel + dkv_kernel + depth_cols_kernel",
+        launches = ["fwd_kernel", "dq_kernel"] + (["dkv_kernel"] if mode != "depth_only" else []) + ([depth_kernel] if depth_kernel else [])
+        roofline = {"bound": "hbm", "kernel": " + ".join(launches),
                     "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                     "algorithmic_bytes": mb, "traffic": whole,
                     "traffic_source": "profiles/hbm_traffic.json (recorded)" if whole is not None else None}

@@ -145,9 +145,12 @@ int moda_hip_fwd(const moda_hip_desc* desc, const void* q, const void* k, const 
  * o * do of moda_v14.py:525-539, kept in a form private to the library) and, for launches whose key
  * tiles alone would leave compute units idle, fp32 partial sums of dk, dv per row segment (the role of
  * the reference's dk_grouped / dv_grouped buffers, moda_v14.py:1715-1752; added up in a fixed order).
+ * Outside chunk-visible mode (head dims up to 128) it also holds the rounded probabilities and dS of every
+ * (query row, depth slot) pair, 2 * 2 bytes each, which the dQ kernel leaves for the launch that forms dkd, dvd.
  * A smaller workspace is accepted down to the row sums alone (B * H * G * T * 4 bytes; packed batch:
  * H * G * total_tokens * 4): the backward then uses fewer row segments or none, which changes the fp32
- * summation order of dk, dv but nothing else.  Returns 0 for an invalid descriptor.
+ * summation order of dk, dv, and recomputes the depth scores in the depth-gradient launch (fp32 dot products
+ * in place of the matrix products: the same values up to fp32 rounding).  Returns 0 for an invalid descriptor.
  */
 size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* desc);
 /* `workspace` below must be 4-byte aligned (MODA_HIP_EALIGN otherwise); the row segments are only used when it is

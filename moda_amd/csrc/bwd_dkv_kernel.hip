@@ -724,6 +724,161 @@ __global__ __launch_bounds__(256) void depth_cols_kernel(const KArgs a_in) {
   if (in_v) *reinterpret_cast<i32x4*>(dv_out) = ov;
 }
 
+// The same columns when the dQ kernel has left its rounded P and dS of every (query row, slot) pair in the workspace
+// (KArgs::depth_p, depth_ds): no kd, vd, no scores -- per column G scalar pairs and the G rows of q and do, which the
+// L columns of a token share through the caches.  The launch moves the gradient rows out and little else.
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void depth_cols_handed_kernel(const KArgs a_in) {
+  constexpr int LPC = HD / 8, CPW = 64 / LPC, CPB = 4 * CPW;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = lane % LPC;
+  KArgs a = a_in;
+  const int BHk = a.B * a.Hkv;
+  const int bh = blockIdx.x % BHk;
+  int b = bh / a.Hkv;
+  const int hkv = bh % a.Hkv;
+  enter_sequence(a, b);
+  const int64_t c = (int64_t)(blockIdx.x / BHk) * CPB + wave * CPW + lane / LPC;
+  if (c >= (int64_t)a.T * a.L) return;  // whole lane groups leave together
+  const int w = (int)(c / a.L), slot = (int)(c - (int64_t)w * a.L);
+  uint16_t* dk_out = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + c * a.sdkd.t + 8 * sub;
+  uint16_t* dv_out = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + c * a.sdvd.t + 8 * sub;
+  const bool in_k = 8 * sub < a.D, in_v = 8 * sub < a.Dv;
+  if (slot >= a.Lv) {  // a slot without data: zero gradient, or (accumulating) somebody else's sum to leave alone
+    if (a.accum_depth) return;
+    const i32x4 z = {0, 0, 0, 0};
+    if (in_k) *reinterpret_cast<i32x4*>(dk_out) = z;
+    if (in_v) *reinterpret_cast<i32x4*>(dv_out) = z;
+    return;
+  }
+  auto load8 = [&](const uint16_t* p, float (&f)[8], bool in_dim) {
+    const i32x4 zero = {0, 0, 0, 0};
+    const i32x4 v = in_dim ? *reinterpret_cast<const i32x4*>(p) : zero;
+#pragma unroll
+    for (int i = 0; i < 4; i++) unpack2<T>(v[i], f[2 * i], f[2 * i + 1]);
+  };
+  float dk[8], dv[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) dk[i] = dv[i] = 0.f;
+  const uint16_t* qb = a.q + b * a.sq.b + hkv * a.sq.h + 8 * sub;
+  const uint16_t* dob = a.d_o + b * a.sdo.b + hkv * a.sdo.h + 8 * sub;
+  const int64_t head = ((int64_t)b * a.Hq + hkv) * a.delta_pitch;
+  for (int gq = 0; gq < a.Gf; gq++) {
+    const int64_t r = (int64_t)w * a.Gf + gq;
+    float qf[8], dof[8];
+    load8(qb + r * a.sq.t, qf, in_k);
+    load8(dob + r * a.sdo.t, dof, in_v);
+    float p, ds, unused;
+    const int64_t at = (head + (int64_t)w * a.Gf) * a.Lv + (int64_t)slot * a.Gf + gq;
+    unpack2<T>((int)a.depth_p[at], p, unused);
+    unpack2<T>((int)a.depth_ds[at], ds, unused);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      dv[i] = __builtin_fmaf(p, dof[i], dv[i]);
+      dk[i] = __builtin_fmaf(ds, qf[i], dk[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) dk[i] *= a.scale;
+  if (a.accum_depth) {  // add to what the row holds (this thread is its only writer), one rounding per call
+    float ok_old[8], ov_old[8];
+    load8(dk_out, ok_old, in_k);
+    load8(dv_out, ov_old, in_v);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      dk[i] += ok_old[i];
+      dv[i] += ov_old[i];
+    }
+  }
+  i32x4 ok, ov;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    ok[i] = pack2<T>(dk[2 * i], dk[2 * i + 1]);
+    ov[i] = pack2<T>(dv[2 * i], dv[2 * i + 1]);
+  }
+  if (in_k) *reinterpret_cast<i32x4*>(dk_out) = ok;
+  if (in_v) *reinterpret_cast<i32x4*>(dv_out) = ov;
+}
+
+// The same for query groups of up to four rows, organised by token: the lanes that share a token (16 bytes of the head
+// dim each) keep the token's rows of q and do in registers and walk its slots, so that q and do are read once per
+// token instead of once per slot and the launch is little more than the stream of gradient rows going out.
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void depth_token_handed_kernel(const KArgs a_in) {
+  constexpr int LPT = HD / 8, TPW = 64 / LPT, TPB = 4 * TPW, GMAX = 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = lane % LPT;
+  KArgs a = a_in;
+  const int BHk = a.B * a.Hkv;
+  const int bh = blockIdx.x % BHk;
+  int b = bh / a.Hkv;
+  const int hkv = bh % a.Hkv;
+  enter_sequence(a, b);
+  const int w = (blockIdx.x / BHk) * TPB + wave * TPW + lane / LPT;
+  if (w >= a.T) return;  // whole lane groups leave together
+  const bool in_k = 8 * sub < a.D, in_v = 8 * sub < a.Dv;
+  auto load8 = [&](const uint16_t* p, float (&f)[8], bool in_dim) {
+    const i32x4 zero = {0, 0, 0, 0};
+    const i32x4 v = in_dim ? *reinterpret_cast<const i32x4*>(p) : zero;
+#pragma unroll
+    for (int i = 0; i < 4; i++) unpack2<T>(v[i], f[2 * i], f[2 * i + 1]);
+  };
+  float qf[GMAX][8], dof[GMAX][8];
+  const uint16_t* qb = a.q + b * a.sq.b + hkv * a.sq.h + 8 * sub;
+  const uint16_t* dob = a.d_o + b * a.sdo.b + hkv * a.sdo.h + 8 * sub;
+#pragma unroll
+  for (int g = 0; g < GMAX; g++) {
+    const int64_t r = (int64_t)w * a.Gf + g;
+    load8(qb + r * a.sq.t, qf[g], in_k && g < a.Gf);
+    load8(dob + r * a.sdo.t, dof[g], in_v && g < a.Gf);
+  }
+  const int64_t block = (((int64_t)b * a.Hq + hkv) * a.delta_pitch + (int64_t)w * a.Gf) * a.Lv;
+  uint16_t* dk_out = a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + (int64_t)w * a.L * a.sdkd.t + 8 * sub;
+  uint16_t* dv_out = a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + (int64_t)w * a.L * a.sdvd.t + 8 * sub;
+  for (int slot = 0; slot < a.L; slot++, dk_out += a.sdkd.t, dv_out += a.sdvd.t) {
+    float dk[8], dv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) dk[i] = dv[i] = 0.f;
+    if (slot >= a.Lv) {  // a slot without data: zero gradient, or (accumulating) somebody else's sum to leave alone
+      if (a.accum_depth) continue;
+    } else {
+#pragma unroll
+      for (int g = 0; g < GMAX; g++) {
+        float p = 0.f, ds = 0.f, unused;
+        if (g < a.Gf) {
+          unpack2<T>((int)a.depth_p[block + (int64_t)slot * a.Gf + g], p, unused);
+          unpack2<T>((int)a.depth_ds[block + (int64_t)slot * a.Gf + g], ds, unused);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          dv[i] = __builtin_fmaf(p, dof[g][i], dv[i]);
+          dk[i] = __builtin_fmaf(ds, qf[g][i], dk[i]);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; i++) dk[i] *= a.scale;
+      if (a.accum_depth) {  // add to what the row holds (this thread is its only writer), one rounding per call
+        float ok_old[8], ov_old[8];
+        load8(dk_out, ok_old, in_k);
+        load8(dv_out, ov_old, in_v);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          dk[i] += ok_old[i];
+          dv[i] += ov_old[i];
+        }
+      }
+    }
+    i32x4 ok, ov;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      ok[i] = pack2<T>(dk[2 * i], dk[2 * i + 1]);
+      ov[i] = pack2<T>(dv[2 * i], dv[2 * i + 1]);
+    }
+    if (in_k) *reinterpret_cast<i32x4*>(dk_out) = ok;
+    if (in_v) *reinterpret_cast<i32x4*>(dv_out) = ov;
+  }
+}
+
 // A partially filled depth stream, not accumulating: the chunk-visible kernels above, and the dQ kernel where it
 // forms the depth gradients itself, only visit the slots that hold data, so the gradient rows of the other slots
 // are written here (zeros).  One thread per 16 bytes of a
@@ -847,7 +1002,18 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
     constexpr int CPB = 4 * (64 / (HD / 8));
     const int64_t nx = (((int64_t)a.T * a.L + CPB - 1) / CPB) * a.B * a.Hkv;
     if (nx >= (1ll << 31)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((depth_cols_kernel<T, HD>), dim3((unsigned)nx), dim3(256), 0, stream, a);
+    if constexpr (HD <= 128) {
+      if (a.depth_p && a.Gf <= 4) {
+        constexpr int TPB = 4 * (64 / (HD / 8));
+        const int64_t nt = (((int64_t)a.T + TPB - 1) / TPB) * a.B * a.Hkv;
+        hipLaunchKernelGGL((depth_token_handed_kernel<T, HD>), dim3((unsigned)nt), dim3(256), 0, stream, a);
+      } else if (a.depth_p)
+        hipLaunchKernelGGL((depth_cols_handed_kernel<T, HD>), dim3((unsigned)nx), dim3(256), 0, stream, a);
+      else
+        hipLaunchKernelGGL((depth_cols_kernel<T, HD>), dim3((unsigned)nx), dim3(256), 0, stream, a);
+    } else {
+      hipLaunchKernelGGL((depth_cols_kernel<T, HD>), dim3((unsigned)nx), dim3(256), 0, stream, a);
+    }
   }
   return hipGetLastError();
 }

@@ -206,8 +206,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   for (int nb = 0; nb < NB; nb++) dp_init[nb] = f32x4{delta[nb], delta[nb], delta[nb], delta[nb]};
   // `nblk`: 16-column blocks of the tile (4, or 2 for a wave's own depth tiles); `scored` runs once K and V
   // have been read for the scores (V is not needed after that)
+  // `emit(mb, nb, p, ds)`: called with the probabilities and the dS of every 4-column piece (the wave's own depth
+  // tiles use it to hand them to the depth-gradient kernel)
   auto tile = [&](auto masked, auto nblk, lds_cptr Kc, lds_cptr Vc, int col0, const int (&lo)[NB], const int (&hi)[NB],
-                  auto&& scored) {
+                  auto&& scored, auto&& emit) {
     constexpr bool MASKED = decltype(masked)::value;
     constexpr int MBLK = decltype(nblk)::value;
     f32x4 s[MBLK][NB], dp[MBLK][NB];
@@ -218,7 +220,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
 #pragma unroll
     for (int mb = 0; mb < MBLK; mb++)
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
+      for (int nb = 0; nb < NB; nb++) {
+        f32x4 pr;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           float p = fast_exp2(__builtin_fmaf(s[mb][nb][i], sc, -lse[nb]));
@@ -226,8 +229,11 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
             const int c = col0 + 16 * mb + slot_base(q4) + i;
             p = (c >= lo[nb] && c < hi[nb]) ? p : 0.f;
           }
+          pr[i] = p;
           s[mb][nb][i] = p * dp[mb][nb][i];
         }
+        emit(mb, nb, pr, s[mb][nb]);
+      }
     i32x4 DS[MBLK / 2][NB];
 #pragma unroll
     for (int ks = 0; ks < MBLK / 2; ks++)
@@ -244,7 +250,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
   for (; it < n_full; it++) {
     if (it + DIST < ntiles) issue(it + DIST);
     lds_cptr Kc = smem + c_st * 2 * BN * HD;
-    tile(std::false_type{}, four, Kc, Kc + BN * HD, it * BN, none, none, []() {});
+    tile(std::false_type{}, four, Kc, Kc + BN * HD, it * BN, none, none, []() {}, [](int, int, const f32x4&, const f32x4&) {});
     c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
     wait_tile(it + 1);
     __syncthreads();
@@ -263,7 +269,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
     }
     if (__any(touches)) {
       lds_cptr Kc = smem + c_st * 2 * BN * HD;
-      tile(std::true_type{}, four, Kc, Kc + BN * HD, col0, lo, hi, []() {});
+      tile(std::true_type{}, four, Kc, Kc + BN * HD, col0, lo, hi, []() {}, [](int, int, const f32x4&, const f32x4&) {});
     }
     c_st = (c_st + 1 == NST) ? 0 : c_st + 1;
     wait_tile(it + 1);
@@ -304,14 +310,40 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
       fetch(Kt, kdp, a.skd.t, c_beg, a.D);
       fetch(Vt, vdp, a.svd.t, c_beg, a.Dv);
       const std::integral_constant<int, 2> two{};
+      // where the depth-gradient kernel takes P and dS from here: this lane's rows of the two arrays
+      const bool hand_over = a.depth_p != nullptr;
+      uint16_t *hp[NB], *hds[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        const int r = rw0 + 16 * nb + n, t = r / a.Gf;  // slot l of row r: element l * Gf + (r - t * Gf) of token t's block
+        const int64_t at = (((int64_t)b * a.Hq + hq) * (VARLEN ? a.delta_pitch : a.Tq) + (int64_t)t * a.Gf) * a.Lv + (r - t * a.Gf);
+        hp[nb] = a.depth_p + at;
+        hds[nb] = a.depth_ds + at;
+      }
       for (int j = 0; j < nh; j++) {
         const int col0 = c_beg + 32 * j;
         const bool more = j + 1 < nh;
         Own::template wait_but<0>();
-        tile(std::true_type{}, two, Kt, Vt, col0, dlo, dhi, [&]() {
-          Own::reads_done();
-          if (more) fetch(Vt, vdp, a.svd.t, col0 + 32, a.Dv);
-        });
+        tile(std::true_type{}, two, Kt, Vt, col0, dlo, dhi,
+             [&]() {
+               Own::reads_done();
+               if (more) fetch(Vt, vdp, a.svd.t, col0 + 32, a.Dv);
+             },
+             [&](int mb, int nb, const f32x4& p, const f32x4& ds) {
+               if (!hand_over) return;
+               // rounded as the matrix products take them; slot of column c within its row: c - dlo
+               const int w0 = pack2<T>(p[0], p[1]), w1 = pack2<T>(p[2], p[3]);
+               const int x0 = pack2<T>(ds[0], ds[1]), x1 = pack2<T>(ds[2], ds[3]);
+#pragma unroll
+               for (int i = 0; i < 4; i++) {
+                 const int c = col0 + 16 * mb + slot_base(q4) + i;
+                 if (c >= dlo[nb] && c < dhi[nb]) {
+                   const int pw = (i < 2) ? w0 : w1, dw = (i < 2) ? x0 : x1;
+                   hp[nb][(c - dlo[nb]) * a.Gf] = (uint16_t)((i & 1) ? ((unsigned)pw >> 16) : ((unsigned)pw & 0xffffu));
+                   hds[nb][(c - dlo[nb]) * a.Gf] = (uint16_t)((i & 1) ? ((unsigned)dw >> 16) : ((unsigned)dw & 0xffffu));
+                 }
+               }
+             });
         Own::reads_done();
         if (more) fetch(Kt, kdp, a.skd.t, col0 + 32, a.D);
       }

@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include "../../include/moda_hip.h"
+#include "geometry.h"
 #include "kargs.h"
 
 namespace moda {
@@ -143,6 +144,14 @@ int desired_dkv_split(const moda_hip_desc* d, const KArgs& a) {
   int s = 1;
   while (tiles * s < 512 && s < 8 && query_tiles / (2 * s) >= 16) s *= 2;
   return s;
+}
+
+// P and dS of the (query row, depth slot) pairs, handed from the dQ kernel to the depth-gradient kernel (see
+// KArgs::depth_p): two 16-bit arrays indexed like the row sums, times the slots that hold data.
+size_t depth_handover_bytes(const moda_hip_desc* d, const KArgs& a) {
+  if (!use_mfma(d) || !moda::depth_scores_from_dq(a, tile_width(d))) return 0;
+  const size_t n = (a.cu ? (size_t)1 : (size_t)a.B) * a.Hq * a.delta_pitch * a.Lv * sizeof(uint16_t);
+  return 2 * ((n + 255) / 256 * 256);
 }
 
 size_t dkv_part_bytes(const moda_hip_desc* d, const KArgs& a, int split) {
@@ -288,7 +297,9 @@ size_t moda_hip_bwd_workspace_bytes(const moda_hip_desc* d) {
   KArgs a;
   if (fill_geometry(d, a)) return 0;
   const size_t part = dkv_part_bytes(d, a, desired_dkv_split(d, a));
-  return part ? delta_bytes(a) + part : delta_bytes_exact(a);  // packed batches: the row sums only
+  const size_t hand = depth_handover_bytes(d, a);
+  // the row sums, then (each optional) the handed-over depth scores and the partial sums of the row split
+  return (part || hand) ? delta_bytes(a) + hand + part : delta_bytes_exact(a);
 }
 
 int moda_hip_bwd(const moda_hip_desc* d, const void* q, const void* k, const void* v, const void* kd,
@@ -378,11 +389,19 @@ int moda_hip_bwd_stages(const moda_hip_desc* d, const void* q, const void* k, co
     if ((uintptr_t)workspace % sizeof(float) != 0) return MODA_HIP_EALIGN;
     // the row split of light launches uses what the workspace offers beyond the row sums: a caller that gives
     // less than moda_hip_bwd_workspace_bytes asks for (moda_hip_bwd_static) gets fewer segments or none
+    // ... and likewise the hand-over of the depth scores from the dQ kernel to the depth-gradient kernel, which sits
+    // between the row sums and the partial sums
+    size_t hand = depth_handover_bytes(d, a);
+    if (delta_bytes(a) + hand > workspace_bytes) hand = 0;
     int split = desired_dkv_split(d, a);
-    while (split > 1 && delta_bytes(a) + dkv_part_bytes(d, a, split) > workspace_bytes) split /= 2;
+    while (split > 1 && delta_bytes(a) + hand + dkv_part_bytes(d, a, split) > workspace_bytes) split /= 2;
     if ((uintptr_t)workspace % 16 != 0) split = 1;  // the partial sums are written and read 16 bytes at a time
     a.dkv_split = split;
-    a.dkv_part = (float*)((char*)workspace + delta_bytes(a));
+    a.dkv_part = (float*)((char*)workspace + delta_bytes(a) + hand);
+    if (hand) {
+      a.depth_p = (uint16_t*)((char*)workspace + delta_bytes(a));
+      a.depth_ds = (uint16_t*)((char*)workspace + delta_bytes(a) + hand / 2);
+    }
   } else {
     return MODA_HIP_OK;
   }

@@ -67,6 +67,14 @@ MODA_HD bool depth_grads_in_dq(const KArgs& a, int HD) {
   return a.L > 0 && !a.chunk && HD <= kDepthGradsInDqMaxWidth && 32 % a.Gf == 0;
 }
 
+// ... and where the dQ kernel's waves walk their own depth columns without forming the gradients (the 128-wide tiles,
+// or a query group that does not divide a wave), they can at least hand their rounded P and dS of the (row, slot)
+// pairs to the depth-column kernel through the workspace (KArgs::depth_p), which then skips reading kd, vd and
+// recomputing the scores.
+MODA_HD bool depth_scores_from_dq(const KArgs& a, int HD) {
+  return a.L > 0 && !a.chunk && HD <= 128 && !depth_grads_in_dq(a, HD);
+}
+
 // The column tiles of query tile qt: n_seq sequence tiles, of which the first n_full are seen completely by every
 // row of the workgroup, then n_dep depth tiles starting at flattened depth column dep0 (ring_depth: the depth
 // columns go through the ring at all).

@@ -28,6 +28,12 @@ struct KArgs {
   int has_seq, causal, chunk;
   int accum_depth;  // dkd, dvd += (slots l >= Lv untouched) instead of = (slots l >= Lv zeroed)
   int own_delta;    // the dQ kernel forms the row sums of o * do itself and leaves them in `delta` for the later kernels
+  // Outside chunk-visible mode a query row sees the Lv depth slots of its own token only.  When the dQ kernel walks
+  // them (its waves' own depth columns) it leaves the rounded P and dS of those (row, slot) pairs here,
+  // [B, Hq, delta_pitch / Gf tokens, Lv, Gf] each (a token's block starts at the `delta` index of its first row
+  // times Lv; inside it slot-major, the token's Gf rows side by side), and the depth-gradient kernel forms dkd, dvd
+  // from them and the rows of q, do without reading kd, vd again.  Null: no room in the workspace, or another route.
+  uint16_t *depth_p, *depth_ds;
   // Sequence dK/dV of launches too small to fill the device: the query rows of every column tile are cut into
   // `dkv_split` segments, one workgroup each, which leave fp32 partial sums in `dkv_part`
   // ([2 (dk, dv)][dkv_split][B][Hkv][T][D]); a second kernel adds them in segment order.  1 = no split.
@@ -66,6 +72,10 @@ __host__ __device__ __forceinline__ void enter_sequence(KArgs& a, int& b, int un
   a.dvd += c0 * a.sdvd.t;
   a.lse += (int64_t)t0 * a.Gf * a.Hq;
   a.delta += (int64_t)t0 * a.Gf;
+  if (a.depth_p) {
+    a.depth_p += (int64_t)t0 * a.Gf * a.Lv;
+    a.depth_ds += (int64_t)t0 * a.Gf * a.Lv;
+  }
   a.T = T;
   a.Tq = T * a.Gf;
   b = 0;

@@ -178,6 +178,11 @@ KArgs make_args(const Case& c) {
   a.dvd = (uint16_t*)add_region("dvd", idx++, bytes((int64_t)T * c.L, c.H, c.Dv), 2, true);
   a.lse = (float*)add_region("lse", idx++, (uint64_t)Bt * qrows * a.Hq * 4, 4, true);
   a.delta = (float*)add_region("delta", idx++, (uint64_t)(c.packed ? 1 : c.nseq) * a.Hq * a.delta_pitch * 4, 4, true);
+  if (depth_scores_from_dq(a, c.HD)) {  // P and dS of the (query row, slot) pairs, handed from dQ to the depth-gradient kernel
+    const uint64_t n = (uint64_t)(c.packed ? 1 : c.nseq) * a.Hq * a.delta_pitch * a.Lv * 2;
+    a.depth_p = (uint16_t*)add_region("hand_p", idx++, n, 2, true);
+    a.depth_ds = (uint16_t*)add_region("hand_ds", idx++, n, 2, true);
+  }
   a.sq = a.sdq = strides(qrows, a.Hq, c.D);
   a.so = a.sdo = strides(qrows, a.Hq, c.Dv);
   a.sk = a.sdk = strides(T, c.H, c.D);
@@ -345,6 +350,26 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
               check_dma("vd", a.vd + b * a.svd.b + hkv * a.svd.h + (int64_t)col0 * a.svd.t,
                         nrows > 0 ? (uint32_t)nrows * (uint32_t)a.svd.t * 2u : 0u, voffv, 0, 16, vt + set + i * 1024, lds_bytes,
                         voffv == kPadOffset);
+            }
+          }
+          // dQ kernel handing P and dS of its rows' visible depth columns to the depth-gradient kernel: lane (n, q4)
+          // holds, per 16-column block, the columns slot_base(q4) .. +3 of rows 16*nb + n
+          if (dq && a.depth_p && !depth_grads_in_dq(a, HD)) {
+            const int n = lane & 15, q4 = lane >> 4;
+            ctx(kname, (int)block, wave, lane, "depth scores for the depth-gradient kernel");
+            for (int nb = 0; nb < rows_per_wave / 16; nb++) {
+              const int r = rw0 + 16 * nb + n;
+              const RowVis vis = row_visibility(a, r, Ld);
+              const int t = r / a.Gf;  // slot l of row r: element l * Gf + (r - t * Gf) of token t's block
+              const int64_t at = (((int64_t)b * a.Hq + hq) * (varlen ? a.delta_pitch : a.Tq) + (int64_t)t * a.Gf) * a.Lv + (r - t * a.Gf);
+              for (int j = 0; j < nh; j++)
+                for (int mb = 0; mb < 2; mb++)
+                  for (int i = 0; i < 4; i++) {
+                    const int c = span.c_beg + 32 * j + 16 * mb + slot_base(q4) + i;
+                    if (c < vis.dlo || c >= vis.dhi) continue;
+                    check_access("hand_p", a.depth_p + at + (int64_t)(c - vis.dlo) * a.Gf, 2, true);
+                    check_access("hand_ds", a.depth_ds + at + (int64_t)(c - vis.dlo) * a.Gf, 2, true);
+                  }
             }
           }
           // dQ kernel outside chunk-visible mode: the same pass forms dK and dV of the wave's own depth columns.
@@ -640,17 +665,61 @@ void walk_depth_cols(const KArgs& a_in) {
         }
         continue;
       }
-      if (in_k) check_access("kd", a.kd + b * a.skd.b + hkv * a.skd.h + c * a.skd.t + 8 * sub, 16, false);
-      if (in_v) check_access("vd", a.vd + b * a.svd.b + hkv * a.svd.h + c * a.svd.t + 8 * sub, 16, false);
+      const bool handed = a.depth_p != nullptr;  // depth_cols_handed_kernel: P and dS from the dQ kernel, no kd, vd, statistics
+      if (!handed && in_k) check_access("kd", a.kd + b * a.skd.b + hkv * a.skd.h + c * a.skd.t + 8 * sub, 16, false);
+      if (!handed && in_v) check_access("vd", a.vd + b * a.svd.b + hkv * a.svd.h + c * a.svd.t + 8 * sub, 16, false);
       for (int gq = 0; gq < a.Gf; gq++) {
         const int64_t r = (int64_t)w * a.Gf + gq;
         if (in_k) check_access("q", a.q + b * a.sq.b + hkv * a.sq.h + 8 * sub + r * a.sq.t, 16, false);
         if (in_v) check_access("do", a.d_o + b * a.sdo.b + hkv * a.sdo.h + 8 * sub + r * a.sdo.t, 16, false);
+        if (handed) {
+          const int64_t at = (((int64_t)b * a.Hq + hkv) * a.delta_pitch + (int64_t)w * a.Gf) * a.Lv + (int64_t)slot * a.Gf + gq;
+          check_access("hand_p", a.depth_p + at, 2, false);
+          check_access("hand_ds", a.depth_ds + at, 2, false);
+          continue;
+        }
         check_access("lse", a.lse + ((int64_t)b * a.Tq + r) * a.Hq + hkv, 4, false);
         check_access("delta", a.delta + ((int64_t)b * a.Hq + hkv) * a.delta_pitch + r, 4, false);
       }
       if (in_k) check_access("dkd", dk_out, 16, true);
       if (in_v) check_access("dvd", dv_out, 16, true);
+    }
+}
+
+// the same organised by token (query groups of up to four rows with the depth scores handed over by the dQ kernel)
+template <int HD>
+void walk_depth_tokens(const KArgs& a_in) {
+  constexpr int LPT = HD / 8, TPW = 64 / LPT, TPB = 4 * TPW;
+  const int BHk = a_in.B * a_in.Hkv;
+  const int64_t nt = (((int64_t)a_in.T + TPB - 1) / TPB) * BHk;
+  for (int64_t block = 0; block < nt; block++)
+    for (int tid = 0; tid < 256; tid++) {
+      const int lane = tid & 63, wave = tid >> 6, sub = lane % LPT;
+      const int bh = (int)(block % BHk);
+      int b = bh / a_in.Hkv;
+      const int hkv = bh % a_in.Hkv;
+      const KArgs a = seq_args(a_in, b);
+      const int w = (int)(block / BHk) * TPB + wave * TPW + lane / LPT;
+      if (w >= a.T) continue;
+      const bool in_k = 8 * sub < a.D, in_v = 8 * sub < a.Dv;
+      ctx("depth_token_handed_kernel", (int)block, wave, lane, "token");
+      for (int g = 0; g < a.Gf; g++) {
+        const int64_t r = (int64_t)w * a.Gf + g;
+        if (in_k) check_access("q", a.q + b * a.sq.b + hkv * a.sq.h + 8 * sub + r * a.sq.t, 16, false);
+        if (in_v) check_access("do", a.d_o + b * a.sdo.b + hkv * a.sdo.h + 8 * sub + r * a.sdo.t, 16, false);
+      }
+      const int64_t blk = (((int64_t)b * a.Hq + hkv) * a.delta_pitch + (int64_t)w * a.Gf) * a.Lv;
+      for (int slot = 0; slot < a.L; slot++) {
+        if (slot >= a.Lv && a.accum_depth) continue;
+        if (slot < a.Lv)
+          for (int g = 0; g < a.Gf; g++) {
+            check_access("hand_p", a.depth_p + blk + (int64_t)slot * a.Gf + g, 2, false);
+            check_access("hand_ds", a.depth_ds + blk + (int64_t)slot * a.Gf + g, 2, false);
+          }
+        const int64_t c = (int64_t)w * a.L + slot;
+        if (in_k) check_access("dkd", a.dkd + b * a.sdkd.b + hkv * a.sdkd.h + c * a.sdkd.t + 8 * sub, 16, true);
+        if (in_v) check_access("dvd", a.dvd + b * a.sdvd.b + hkv * a.sdvd.h + c * a.sdvd.t + 8 * sub, 16, true);
+      }
     }
 }
 
@@ -707,6 +776,10 @@ void walk_all(const Case& c, const KArgs& a) {
   }
   require_full("dq");
   require_full("delta");
+  if (a.depth_p) {
+    require_full("hand_p");
+    require_full("hand_ds");
+  }
   walk_dkv<HD>(a);
   if (a.dkv_split > 1 && a.has_seq) {
     require_full("part");
@@ -723,7 +796,10 @@ void walk_all(const Case& c, const KArgs& a) {
         if (depth_by_chunks(a, HD)) walk_chunk_depth<HD>(a);
       }
     } else if (!depth_grads_in_dq(a, HD)) {
-      walk_depth_cols<HD>(a);
+      if (a.depth_p && a.Gf <= 4)
+        walk_depth_tokens<HD>(a);
+      else
+        walk_depth_cols<HD>(a);
     }
     require_full("dkd");
     require_full("dvd");

@@ -54,15 +54,23 @@ def check(name, got, ref, dtype, what=""):
             f"at ref={ref.flatten()[i]:.4e} (atol={atol}, rtol={rtol}); max_abs={err.max():.4e}")
 
 
-def run_hip(inp, scale, G, mode, cb=0, row_sums_only=False):
+def run_hip(inp, scale, G, mode, cb=0, row_sums_only=False, no_row_split=False):
     """``row_sums_only``: give the backward a workspace that holds the row sums and nothing else, which keeps the
-    sequence dK/dV on the single-pass summation order (no row segments)."""
+    sequence dK/dV on the single-pass summation order (no row segments) and the depth gradients on the kernel that
+    recomputes its scores.  ``no_row_split``: a workspace with room for the row sums and the depth scores the dQ kernel
+    hands to the depth-gradient kernel, but not for partial sums (what a packed batch is given)."""
     from moda_amd import ops
 
     m = MODE_ID[mode]
     o, lse = ops._raw_fwd(m, inp["q"], inp["k"], inp["v"], inp["kd"], inp["vd"], scale, G, cb)
-    ws = torch.empty(max(4, 4 * inp["q"].shape[0] * inp["q"].shape[1] * inp["q"].shape[2]), dtype=torch.uint8,
-                     device=inp["q"].device) if row_sums_only else None
+    rows = inp["q"].shape[0] * inp["q"].shape[1] * inp["q"].shape[2]
+    ws = None
+    if row_sums_only:
+        ws = torch.empty(max(4, 4 * rows), dtype=torch.uint8, device=inp["q"].device)
+    elif no_row_split:
+        up = lambda n: (n + 255) // 256 * 256
+        slots = 0 if inp["kd"] is None else inp["kd"].shape[1] // (inp["q"].shape[1] // G)
+        ws = torch.empty(up(4 * rows) + 2 * up(2 * rows * slots), dtype=torch.uint8, device=inp["q"].device)
     dq, dk, dv, dkd, dvd = ops._raw_bwd(m, inp["q"], inp["k"], inp["v"], inp["kd"], inp["vd"], o, lse, inp["do"],
                                         scale, G, cb, ws=ws)
     return {"o": o, "lse": lse, "dq": dq, "dk": dk, "dv": dv, "dkd": dkd, "dvd": dvd}
@@ -1061,7 +1069,7 @@ def test_packed_batch_equals_separate_calls_bitwise(gpu_device):
         part = {n: inp[n][:, a * m:b * m] for n, m in mult.items()}
         part["do"] = inp["do"][:, a * G:b * G]
         # (the packed launch sums dk, dv in one pass per key tile: ask the separate calls for the same order)
-        one = run_hip(part, D ** -0.5, G, "causal", row_sums_only=True)
+        one = run_hip(part, D ** -0.5, G, "causal", no_row_split=True)
         assert torch.equal(o[:, a * G:b * G], one["o"]) and torch.equal(lse[:, a * G:b * G], one["lse"]), i
         for n, key in (("q", "dq"), ("k", "dk"), ("v", "dv"), ("kd", "dkd"), ("vd", "dvd")):
             assert torch.equal(leaf[n].grad[:, a * mult[n]:b * mult[n]], one[key]), (i, n)
