@@ -36,6 +36,8 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
   constexpr int BM = 32 * Shape::W, BN = 64, KK = HD / 16, DB = HD / 32, NT = 64 * Shape::W, NST = Shape::NST,
                 DIST = Shape::DIST;
   constexpr bool PP = Shape::PP;
+  // on the 64-wide tiles the waves' own depth columns go through two sets of private tiles (see the end of the kernel)
+  constexpr bool TWO_OWN_SETS = HD <= 64;
   static_assert(NST >= DIST + 1 + (PP ? 1 : 0) && DIST >= 1 && DIST <= 2,
                 "ring must hold the tile in use, the tiles in flight and (ping-pong) the previous tile");
   static_assert(2 * NST >= Shape::W, "the ring must be large enough for one 32-column K tile and V tile per wave");
@@ -359,6 +361,25 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
       fetch(Kt, kdp, a.skd.t, c_beg, a.D);
       fetch(Vt, vdp, a.svd.t, c_beg, a.Dv);
       const std::integral_constant<int, 1> one{};
+      if constexpr (TWO_OWN_SETS) {
+        // room for two sets of private tiles: the rows of tile j + 1 travel while tile j is worked on
+        constexpr int SET = Shape::W * 2 * 32 * HD;
+        for (int j = 0; j < nh; j++) {
+          const int col0 = c_beg + 32 * j;
+          lds_ptr Kc = Kt + (j & 1) * SET, Vc = Vt + (j & 1) * SET;
+          Own::template wait_but<0>();
+          if (j + 1 < nh) {
+            fetch(Kt + ((j + 1) & 1) * SET, kdp, a.skd.t, col0 + 32, a.D);
+            fetch(Vt + ((j + 1) & 1) * SET, vdp, a.svd.t, col0 + 32, a.Dv);
+          }
+          front(std::true_type{}, one, Kc, col0, dlo, dhi, []() {});
+          TrPipe<T, HD, 2, 2> pv1;
+          const i32x4 P1[2] = {P[0], P[1]};
+          pv1.prefetch(oa, Vc);
+          pv1.run(oa, Vc, P1, o);
+          Own::reads_done();  // this set may be loaded over in the next trip
+        }
+      } else {
       for (int j = 0; j < nh; j++) {
         const int col0 = c_beg + 32 * j;
         const bool more = j + 1 < nh;
@@ -376,6 +397,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_kernel(const KArgs a_in)
         pv1.run(oa, Vt, P1, o);
         Own::reads_done();
         if (more) fetch(Vt, vdp, a.svd.t, col0 + 32, a.Dv);
+      }
       }
     }
   }
@@ -661,7 +683,10 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void fwd_wide_kernel(const KArgs 
 
 template <typename T, int HD, typename Shape, int ADDR>
 hipError_t launch_fwd_t_shape(const KArgs& a, hipStream_t stream) {
-  constexpr size_t smem = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
+  // the ring, or (64-wide tiles) two sets of a private 32-column K tile and V tile per wave, whichever is larger
+  constexpr size_t ring = (size_t)Shape::NST * 2 * 64 * HD * sizeof(uint16_t);
+  constexpr size_t own = HD <= 64 ? (size_t)2 * Shape::W * 2 * 32 * HD * sizeof(uint16_t) : 0;
+  constexpr size_t smem = ring > own ? ring : own;
   static LdsAttrState attr;
   const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&fwd_kernel<T, HD, Shape, ADDR>), smem);
   if (ea != hipSuccess) return ea;

@@ -328,7 +328,8 @@ void walk_row_kernel(const KArgs& a_in, bool dq, int rows_per_wave, bool own_pos
             const int col0 = span.c_beg + 32 * j;
             const int nrows = imin(32, span.c_end - col0);
             // where the dQ kernel forms the depth gradients it alternates between two sets of private tiles
-            const uint32_t set = (dq && depth_grads_in_dq(a, HD)) ? (uint32_t)(j & 1) * Shape::W * 64 * HD * 2 : 0u;
+            // ... and so does the forward kernel on the 64-wide tiles
+            const uint32_t set = ((dq && depth_grads_in_dq(a, HD)) || (!dq && HD <= 64)) ? (uint32_t)(j & 1) * Shape::W * 64 * HD * 2 : 0u;
             for (int i = 0; i < Own::N; i++) {
               if (a.Lv != a.L) {
                 const int w0 = col0 / a.Lv, l0 = col0 - w0 * a.Lv;
@@ -747,13 +748,17 @@ void walk_all(const Case& c, const KArgs& a) {
   const bool small = use_small_rows(a.Tq, (long long)a.B * a.Hq, a.compute_units);
   // ---- forward
   g_ctx = "forward";
+  auto fwd_lds = [&](int W, int NST) {  // the ring, or (64-wide tiles) two sets of private tiles per wave
+    const uint32_t ring = (uint32_t)NST * 2 * 64 * HD * 2, own = HD <= 64 ? 2u * W * 2 * 32 * HD * 2 : 0u;
+    return std::max(ring, own);
+  };
   if constexpr (HD > 128) {
     walk_row_kernel<HD, RowWide, false>(a, false, 16, false, RowWide::NST * 2 * 64 * HD * 2, "fwd_wide_kernel");
   } else {
     if (small)
-      walk_row_kernel<HD, RowSmall<HD>, false>(a, false, 32, true, RowSmall<HD>::NST * 2 * 64 * HD * 2, "fwd_kernel(small)");
+      walk_row_kernel<HD, RowSmall<HD>, false>(a, false, 32, true, fwd_lds(RowSmall<HD>::W, RowSmall<HD>::NST), "fwd_kernel(small)");
     else
-      walk_row_kernel<HD, RowLargePP, false>(a, false, 32, true, RowLargePP::NST * 2 * 64 * HD * 2, "fwd_kernel");
+      walk_row_kernel<HD, RowLargePP, false>(a, false, 32, true, fwd_lds(RowLargePP::W, RowLargePP::NST), "fwd_kernel");
   }
   require_full("o");
   require_full("lse");
