@@ -26,7 +26,9 @@ def walker(tmp_path_factory):
     if shutil.which("hipcc") is None:
         pytest.skip("hipcc not found")
     out = str(tmp_path_factory.mktemp("walker") / "address_walker")
-    subprocess.run(["hipcc", "-x", "hip", "--cuda-host-only", "-std=c++17", "-O1",
+    # host pass only, under AddressSanitizer (the walker's own tables and the kernels' index code run checked)
+    subprocess.run(["hipcc", "-x", "hip", "--cuda-host-only", "-std=c++17", "-O1", "-g", "-fsanitize=address",
+                    "-fno-gpu-sanitize", "-fno-omit-frame-pointer",
                     os.path.join(ROOT, "tests", "address_walker.cpp"), "-o", out], check=True,
                    stdout=subprocess.PIPE, stderr=subprocess.PIPE)
     return out
