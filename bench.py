@@ -441,8 +441,10 @@ def main():
 
         n = max(2, steps // 2)
         t_fwd = ev_time(fwd, n)
+        # the row sums: as a launch of their own (informational), and where a whole backward forms them, inside the
+        # dQ kernel (asked for together with the dQ stage)
         t_delta = ev_time(lambda: bwd(_lib.STAGE_DELTA), n)
-        t_dq = ev_time(lambda: bwd(_lib.STAGE_DQ), n)
+        t_dq = ev_time(lambda: bwd(_lib.STAGE_DELTA | _lib.STAGE_DQ), n)
         t_dkv = ev_time(lambda: bwd(_lib.STAGE_DKV), n)
         Hq = Hkv * G
         if packed is not None:
