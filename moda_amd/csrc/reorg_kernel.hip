@@ -28,14 +28,28 @@ __global__ __launch_bounds__(256) void reorg_kernel(const ReorgArgs a) {
   const int vec_per_row = (int)(a.row_bytes / sizeof(V));
   const int total = vec_per_row * a.n_layers;
   char* cbase = reinterpret_cast<char*>(a.cache) + tok * a.cache_token_bytes + a.slot0_bytes;
-  for (int i = threadIdx.x; i < total; i += 256) {
+  auto at = [&](int i, V*& lp, V*& cp) {
     const int l = i / vec_per_row, w = i - l * vec_per_row;
-    V* lp = reinterpret_cast<V*>(reinterpret_cast<char*>(a.layer[l]) + tok * a.row_bytes) + w;
-    V* cp = reinterpret_cast<V*>(cbase + (int64_t)l * a.row_bytes) + w;
-    if (TO_CACHE)
-      *cp = *lp;
-    else
-      *lp = *cp;
+    lp = reinterpret_cast<V*>(reinterpret_cast<char*>(a.layer[l]) + tok * a.row_bytes) + w;
+    cp = reinterpret_cast<V*>(cbase + (int64_t)l * a.row_bytes) + w;
+  };
+  // Streamed once in, once out: nothing here is read again by this launch.  Four loads go out before the first
+  // store so that a thread keeps 64 bytes in flight.
+  constexpr int U = 4;
+  int i = threadIdx.x;
+  for (; i + (U - 1) * 256 < total; i += U * 256) {
+    V *lp[U], *cp[U], x[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) at(i + u * 256, lp[u], cp[u]);
+#pragma unroll
+    for (int u = 0; u < U; u++) x[u] = __builtin_nontemporal_load(TO_CACHE ? lp[u] : cp[u]);
+#pragma unroll
+    for (int u = 0; u < U; u++) __builtin_nontemporal_store(x[u], TO_CACHE ? cp[u] : lp[u]);
+  }
+  for (; i < total; i += 256) {
+    V *lp, *cp;
+    at(i, lp, cp);
+    __builtin_nontemporal_store(__builtin_nontemporal_load(TO_CACHE ? lp : cp), TO_CACHE ? cp : lp);
   }
 }
 

@@ -27,8 +27,8 @@ def walker(tmp_path_factory):
         pytest.skip("hipcc not found")
     out = str(tmp_path_factory.mktemp("walker") / "address_walker")
     # host pass only, under AddressSanitizer (the walker's own tables and the kernels' index code run checked)
-    subprocess.run(["hipcc", "-x", "hip", "--cuda-host-only", "-std=c++17", "-O1", "-g", "-fsanitize=address",
-                    "-fno-gpu-sanitize", "-fno-omit-frame-pointer",
+    checked = ["-fsanitize=address", "-fno-gpu-sanitize", "-fno-omit-frame-pointer"]  # host code only
+    subprocess.run(["hipcc", "-x", "hip", "--cuda-host-only", "-std=c++17", "-O1", "-g", *checked,
                     os.path.join(ROOT, "tests", "address_walker.cpp"), "-o", out], check=True,
                    stdout=subprocess.PIPE, stderr=subprocess.PIPE)
     return out
