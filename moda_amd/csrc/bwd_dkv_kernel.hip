@@ -526,7 +526,7 @@ __global__ __launch_bounds__(256, 2) void chunk_depth_kernel(const KArgs a_in) {
             val[w] = pack2<T>(x0 + y0, x1 + y1);
           }
         }
-        *dst = val;
+        __builtin_nontemporal_store(val, dst);  // next read by another launch
       }
     }
   };
@@ -874,8 +874,9 @@ __global__ __launch_bounds__(256) void depth_token_handed_kernel(const KArgs a_i
       ok[i] = pack2<T>(dk[2 * i], dk[2 * i + 1]);
       ov[i] = pack2<T>(dv[2 * i], dv[2 * i + 1]);
     }
-    if (in_k) *reinterpret_cast<i32x4*>(dk_out) = ok;
-    if (in_v) *reinterpret_cast<i32x4*>(dv_out) = ov;
+    // written once here and next read by another launch: past the caches
+    if (in_k) __builtin_nontemporal_store(ok, reinterpret_cast<i32x4*>(dk_out));
+    if (in_v) __builtin_nontemporal_store(ov, reinterpret_cast<i32x4*>(dv_out));
   }
 }
 

@@ -449,7 +449,7 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
                   val[w] = pack2<T>(x0 + y0, x1 + y1);
                 }
               }
-              *dst = val;
+              __builtin_nontemporal_store(val, dst);  // next read by another launch
             }
           }
           Own::reads_done();  // the block may be overwritten
