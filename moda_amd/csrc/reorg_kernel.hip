@@ -21,39 +21,64 @@ struct ReorgArgs {
   int n_layers;
 };
 
-// TO_CACHE: layers -> cache; otherwise cache -> layers.
-template <typename V, bool TO_CACHE>
-__global__ __launch_bounds__(256) void reorg_kernel(const ReorgArgs a) {
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+// TO_CACHE: layers -> cache; otherwise cache -> layers.  One workgroup per token.  A thread issues U loads before
+// its first store (the launcher picks the workgroup size and U so that most shapes take one such batch); nothing
+// here is read again by this launch, so both sides bypass the caches' retention.
+template <typename V, bool TO_CACHE, int U, int NT>
+__global__ __launch_bounds__(NT) void reorg_kernel(const ReorgArgs a) {
   const int64_t tok = blockIdx.x;
   const int vec_per_row = (int)(a.row_bytes / sizeof(V));
   const int total = vec_per_row * a.n_layers;
   char* cbase = reinterpret_cast<char*>(a.cache) + tok * a.cache_token_bytes + a.slot0_bytes;
-  auto at = [&](int i, V*& lp, V*& cp) {
+  auto ends = [&](int i, V*& src, V*& dst) {
     const int l = i / vec_per_row, w = i - l * vec_per_row;
-    lp = reinterpret_cast<V*>(reinterpret_cast<char*>(a.layer[l]) + tok * a.row_bytes) + w;
-    cp = reinterpret_cast<V*>(cbase + (int64_t)l * a.row_bytes) + w;
+    V* lp = reinterpret_cast<V*>(reinterpret_cast<char*>(a.layer[l]) + tok * a.row_bytes) + w;
+    V* cp = reinterpret_cast<V*>(cbase + (int64_t)l * a.row_bytes) + w;
+    src = TO_CACHE ? lp : cp;
+    dst = TO_CACHE ? cp : lp;
   };
-  // Streamed once in, once out: nothing here is read again by this launch.  Four loads go out before the first
-  // store so that a thread keeps 64 bytes in flight.
-  constexpr int U = 4;
   int i = threadIdx.x;
-  for (; i + (U - 1) * 256 < total; i += U * 256) {
-    V *lp[U], *cp[U], x[U];
+  for (; i + (U - 1) * NT < total; i += U * NT) {
+    V *src[U], *dst[U], x[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) at(i + u * 256, lp[u], cp[u]);
+    for (int u = 0; u < U; u++) ends(i + u * NT, src[u], dst[u]);
 #pragma unroll
-    for (int u = 0; u < U; u++) x[u] = __builtin_nontemporal_load(TO_CACHE ? lp[u] : cp[u]);
+    for (int u = 0; u < U; u++) x[u] = __builtin_nontemporal_load(src[u]);
 #pragma unroll
-    for (int u = 0; u < U; u++) __builtin_nontemporal_store(x[u], TO_CACHE ? cp[u] : lp[u]);
+    for (int u = 0; u < U; u++) __builtin_nontemporal_store(x[u], dst[u]);
   }
-  for (; i < total; i += 256) {
-    V *lp, *cp;
-    at(i, lp, cp);
-    __builtin_nontemporal_store(__builtin_nontemporal_load(TO_CACHE ? lp : cp), TO_CACHE ? cp : lp);
+  for (; i < total; i += NT) {
+    V *src, *dst;
+    ends(i, src, dst);
+    __builtin_nontemporal_store(__builtin_nontemporal_load(src), dst);
   }
 }
 
-typedef int v4i __attribute__((ext_vector_type(4)));
+template <typename V, bool TO_CACHE, int NT>
+void launch_reorg_batch(const ReorgArgs& a, int64_t n_tokens, int per, hipStream_t stream) {
+  const dim3 grid((unsigned)n_tokens), block(NT);
+  if (per <= 1)
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 1, NT>), grid, block, 0, stream, a);
+  else if (per == 2)
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 2, NT>), grid, block, 0, stream, a);
+  else if (per == 3)
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 3, NT>), grid, block, 0, stream, a);
+  else
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 4, NT>), grid, block, 0, stream, a);
+}
+
+template <typename V, bool TO_CACHE>
+void launch_reorg_kernel(const ReorgArgs& a, int64_t n_tokens, hipStream_t stream) {
+  const int64_t total = a.row_bytes / (int64_t)sizeof(V) * a.n_layers;
+  // 512 threads when that still leaves every thread two accesses, else 256; then as many loads per batch (up to
+  // four) as cover the token in one trip
+  if (total >= 1024)
+    launch_reorg_batch<V, TO_CACHE, 512>(a, n_tokens, (int)((total + 511) / 512), stream);
+  else
+    launch_reorg_batch<V, TO_CACHE, 256>(a, n_tokens, (int)((total + 255) / 256), stream);
+}
 
 hipError_t launch_reorg(void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t n_tokens,
                         int64_t row_bytes, void* cache, bool to_cache, hipStream_t stream) {
@@ -70,17 +95,16 @@ hipError_t launch_reorg(void* const* layers, int64_t n_layers, int64_t slot0, in
     a.slot0_bytes = (slot0 + l0) * row_bytes;
     bool wide = (row_bytes % 16 == 0) && ((uintptr_t)cache % 16 == 0);
     for (int i = 0; i < a.n_layers; i++) wide = wide && ((uintptr_t)a.layer[i] % 16 == 0);
-    const dim3 grid((unsigned)n_tokens), block(256);
     if (wide) {
       if (to_cache)
-        hipLaunchKernelGGL((reorg_kernel<v4i, true>), grid, block, 0, stream, a);
+        launch_reorg_kernel<v4i, true>(a, n_tokens, stream);
       else
-        hipLaunchKernelGGL((reorg_kernel<v4i, false>), grid, block, 0, stream, a);
+        launch_reorg_kernel<v4i, false>(a, n_tokens, stream);
     } else {
       if (to_cache)
-        hipLaunchKernelGGL((reorg_kernel<uint16_t, true>), grid, block, 0, stream, a);
+        launch_reorg_kernel<uint16_t, true>(a, n_tokens, stream);
       else
-        hipLaunchKernelGGL((reorg_kernel<uint16_t, false>), grid, block, 0, stream, a);
+        launch_reorg_kernel<uint16_t, false>(a, n_tokens, stream);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
