@@ -24,9 +24,9 @@ struct ReorgArgs {
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 // TO_CACHE: layers -> cache; otherwise cache -> layers.  One workgroup per token.  A thread issues U loads before
-// its first store (the launcher picks the workgroup size and U so that most shapes take one such batch); nothing
-// here is read again by this launch, so both sides bypass the caches' retention.
-template <typename V, bool TO_CACHE, int U, int NT>
+// its first store (the launcher picks the workgroup size and U so that most shapes take one such batch).  STREAM:
+// nontemporal accesses on both sides.
+template <typename V, bool TO_CACHE, int U, int NT, bool STREAM>
 __global__ __launch_bounds__(NT) void reorg_kernel(const ReorgArgs a) {
   const int64_t tok = blockIdx.x;
   const int vec_per_row = (int)(a.row_bytes / sizeof(V));
@@ -39,45 +39,64 @@ __global__ __launch_bounds__(NT) void reorg_kernel(const ReorgArgs a) {
     src = TO_CACHE ? lp : cp;
     dst = TO_CACHE ? cp : lp;
   };
+  auto get = [](const V* p) { return STREAM ? __builtin_nontemporal_load(p) : *p; };
+  auto put = [](V x, V* p) {
+    if (STREAM)
+      __builtin_nontemporal_store(x, p);
+    else
+      *p = x;
+  };
   int i = threadIdx.x;
   for (; i + (U - 1) * NT < total; i += U * NT) {
     V *src[U], *dst[U], x[U];
 #pragma unroll
     for (int u = 0; u < U; u++) ends(i + u * NT, src[u], dst[u]);
 #pragma unroll
-    for (int u = 0; u < U; u++) x[u] = __builtin_nontemporal_load(src[u]);
+    for (int u = 0; u < U; u++) x[u] = get(src[u]);
 #pragma unroll
-    for (int u = 0; u < U; u++) __builtin_nontemporal_store(x[u], dst[u]);
+    for (int u = 0; u < U; u++) put(x[u], dst[u]);
   }
   for (; i < total; i += NT) {
     V *src, *dst;
     ends(i, src, dst);
-    __builtin_nontemporal_store(__builtin_nontemporal_load(src), dst);
+    put(get(src), dst);
   }
 }
 
-template <typename V, bool TO_CACHE, int NT>
+template <typename V, bool TO_CACHE, int NT, bool STREAM>
 void launch_reorg_batch(const ReorgArgs& a, int64_t n_tokens, int per, hipStream_t stream) {
   const dim3 grid((unsigned)n_tokens), block(NT);
   if (per <= 1)
-    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 1, NT>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 1, NT, STREAM>), grid, block, 0, stream, a);
   else if (per == 2)
-    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 2, NT>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 2, NT, STREAM>), grid, block, 0, stream, a);
   else if (per == 3)
-    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 3, NT>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 3, NT, STREAM>), grid, block, 0, stream, a);
   else
-    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 4, NT>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((reorg_kernel<V, TO_CACHE, 4, NT, STREAM>), grid, block, 0, stream, a);
 }
 
-template <typename V, bool TO_CACHE>
-void launch_reorg_kernel(const ReorgArgs& a, int64_t n_tokens, hipStream_t stream) {
+// What one launch moves (read + written) against the 256 MB of memory-side cache: a copy that fits stays there for
+// the attention kernels that read the cache next; a larger one would only push itself out, and streams past.
+constexpr int64_t kStreamAboveBytes = 256ll << 20;
+
+template <typename V, bool TO_CACHE, bool STREAM>
+void launch_reorg_sized(const ReorgArgs& a, int64_t n_tokens, hipStream_t stream) {
   const int64_t total = a.row_bytes / (int64_t)sizeof(V) * a.n_layers;
   // 512 threads when that still leaves every thread two accesses, else 256; then as many loads per batch (up to
   // four) as cover the token in one trip
   if (total >= 1024)
-    launch_reorg_batch<V, TO_CACHE, 512>(a, n_tokens, (int)((total + 511) / 512), stream);
+    launch_reorg_batch<V, TO_CACHE, 512, STREAM>(a, n_tokens, (int)((total + 511) / 512), stream);
   else
-    launch_reorg_batch<V, TO_CACHE, 256>(a, n_tokens, (int)((total + 255) / 256), stream);
+    launch_reorg_batch<V, TO_CACHE, 256, STREAM>(a, n_tokens, (int)((total + 255) / 256), stream);
+}
+
+template <typename V, bool TO_CACHE>
+void launch_reorg_kernel(const ReorgArgs& a, int64_t n_tokens, hipStream_t stream) {
+  if (2 * n_tokens * a.n_layers * a.row_bytes > kStreamAboveBytes)
+    launch_reorg_sized<V, TO_CACHE, true>(a, n_tokens, stream);
+  else
+    launch_reorg_sized<V, TO_CACHE, false>(a, n_tokens, stream);
 }
 
 hipError_t launch_reorg(void* const* layers, int64_t n_layers, int64_t slot0, int64_t L_total, int64_t n_tokens,
