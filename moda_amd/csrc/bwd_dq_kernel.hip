@@ -539,7 +539,15 @@ __global__ __launch_bounds__(64 * Shape::W, 2) void dq_kernel(const KArgs a_in) 
         i32x2 w;
         w[0] = pack2<T>(dq[d][nb][0] * a.scale, dq[d][nb][1] * a.scale);
         w[1] = pack2<T>(dq[d][nb][2] * a.scale, dq[d][nb][3] * a.scale);
-        if (16 * d + 4 * q4 < a.D) *reinterpret_cast<i32x2*>(op + 16 * d + 4 * q4) = w;
+        if (16 * d + 4 * q4 < a.D) {
+          i32x2* dst = reinterpret_cast<i32x2*>(op + 16 * d + 4 * q4);
+          // the narrow tiles serve HBM-bound shapes whose depth stream can stay in the memory-side cache between
+          // launches if results written once do not displace it
+          if (HD <= 64)
+            __builtin_nontemporal_store(w, dst);
+          else
+            *dst = w;
+        }
       }
     }
   }
