@@ -92,6 +92,37 @@ def make_device_inputs(B, T, Hkv, G, D, L, mode, dev, seed=0):
     return q, k, v, kd, vd, do
 
 
+def bench_fp32_config(dev, steps=20):
+    """The benchmark's fp32 configuration (causal, B=1, T=256, H=Hkv=4, D=64, L=4; the reference's CPU-runnable case):
+    forward + backward on fp32 tensors, in exact fp32 on the vector-ALU kernels (the default) and rounded to fp16
+    operands on the matrix kernels (moda_amd.set_fp32_compute("fp16"))."""
+    import torch
+    from moda_amd import _lib, ops
+
+    B, T, H, D, L = 1, 256, 4, 64, 4
+    gen = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=gen, device=dev, dtype=torch.float32)
+    q, k, v, kd, vd, do = rn(B, T, H, D) * D ** -0.5, rn(B, T, H, D), rn(B, T, H, D), rn(B, T * L, H, D), rn(B, T * L, H, D), rn(B, T, H, D)
+    out = {"workload": f"c1: causal fp32 B={B} T={T} Hq={H} Hkv={H} G=1 D={D} L={L}"}
+    for setting, key in (("fp32", "ms_exact_fp32_vector_alu"), ("fp16", "ms_fp16_operands_matrix_kernels")):
+        previous = ops.set_fp32_compute(setting)
+        try:
+            def step():
+                o, lse = ops._raw_fwd(_lib.CAUSAL, q, k, v, kd, vd, 1.0, 1, 0)
+                ops._raw_bwd(_lib.CAUSAL, q, k, v, kd, vd, o, lse, do, 1.0, 1, 0)
+            for _ in range(3):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            out[key] = (time.perf_counter() - t0) * 1e3 / steps
+        finally:
+            ops.set_fp32_compute(previous)
+    return out
+
+
 def cpu_baseline(B, T, Hkv, G, D, L, mode, cb, target_seconds=15.0):
     """The oracle (torch restatement of the reference's naive MoDA, fp32, forward + backward) timed on the
     host cores on a bounded sample of the same workload: the LAST `tokens` tokens' query rows of ONE
@@ -560,6 +591,7 @@ def main():
                 ttf = 3.5 * t["flops_fwd"] / (t["ms_step"] * 1e-3) / 1e12
                 entry["plain_causal_twin"] = {"ms": t["ms_step"], "tflops": ttf, "moda_over_twin": tf / ttf}
             configs[name] = entry
+        configs["c1"] = bench_fp32_config(dev)
         out["configs"] = configs
         torch.cuda.empty_cache()
     if L > 0:
