@@ -938,6 +938,8 @@ __global__ __launch_bounds__(256) void dkv_reduce_kernel(const KArgs a) {
   }
 }
 
+hipError_t launch_dkv_flat(const KArgs& a, int dtype, hipStream_t stream);  // bwd_dkv_flat_kernel.hip
+
 template <typename T, int HD>
 hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   constexpr int NB = HD > 128 ? 1 : 2, BM = HD > 128 ? 32 : 64, BN = 64 * NB;  // as in dkv_kernel
@@ -958,7 +960,10 @@ hipError_t launch_dkv_t(const KArgs& a, hipStream_t stream) {
   const bool depth_by_chunks = moda::depth_by_chunks(a, HD);
   const int64_t nblk = col_kernel_blocks(a, HD, BN, nseg);
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
-  if (nblk > 0) {
+  if (nblk > 0 && takes_dkv_flat(a, HD, nseg)) {
+    const hipError_t e = launch_dkv_flat(a, std::is_same<T, FP16>::value ? 1 : 0, stream);
+    if (e != hipSuccess) return e;
+  } else if (nblk > 0) {
     if (a.cu)
       hipLaunchKernelGGL((dkv_kernel<T, HD, true>), dim3((unsigned)nblk), dim3(512), smem, stream, a);
     else if (nseg > 1)

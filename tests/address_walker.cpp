@@ -524,6 +524,68 @@ void walk_dkv(const KArgs& a_in) {
   }
 }
 
+// dkv_flat_kernel: four waves, a wave's 32 columns with K and V in registers, query tiles of 32 rows
+template <int HD>
+void walk_dkv_flat(const KArgs& a) {
+  constexpr int NB = 2, BM = 32, BN = 4 * 16 * NB, KS = HD / 32, MB = HD / 16, NST = 3, SP = 64;
+  const uint32_t lds_bytes = 3 * 2 * 32 * HD * 2 + 3 * 2 * 64 * 4;
+  const uint32_t stat_byte = NST * 2 * BM * HD * 2;
+  const int BHk = a.B * a.Hkv;
+  const int64_t nblk = dkv_flat_blocks(a);
+  typedef AsyncTileLoader<HD, BM, 256> Loader;
+  for (int64_t block = 0; block < nblk; block++) {
+    const int bh = (int)(block % BHk), ct = (int)(block / BHk);
+    const int b = bh / a.Hkv, hkv = bh % a.Hkv;
+    const ColTilePlan plan = col_tile_plan(a, a, ct, BN, BM, false, 1);
+    if (!plan.active || plan.dep) fail("dkv_flat_kernel: column tile %d is not a sequence tile", ct);
+    for (int tid = 0; tid < 256; tid++) {
+      const int lane = tid & 63, n = lane & 15, q4 = lane >> 4, wave = tid >> 6;
+      for (int nb = 0; nb < NB; nb++) {
+        const int c = plan.c_first + wave * (16 * NB) + 16 * nb + n;
+        if (c >= a.T) continue;
+        ctx("dkv_flat_kernel", (int)block, wave, lane, "stationary K and V rows");
+        for (int ks = 0; ks < KS; ks++) {
+          if (32 * ks + 8 * q4 < a.D) check_access("k", a.k + b * a.sk.b + hkv * a.sk.h + 8 * q4 + (int64_t)c * a.sk.t + 32 * ks, 16, false);
+          if (32 * ks + 8 * q4 < a.Dv) check_access("v", a.v + b * a.sv.b + hkv * a.sv.h + 8 * q4 + (int64_t)c * a.sv.t + 32 * ks, 16, false);
+        }
+        ctx("dkv_flat_kernel", (int)block, wave, lane, "gradient rows");
+        uint16_t* dkp = a.dk + b * a.sdk.b + hkv * a.sdk.h + (int64_t)c * a.sdk.t + 4 * q4;
+        uint16_t* dvp = a.dv + b * a.sdv.b + hkv * a.sdv.h + (int64_t)c * a.sdv.t + 4 * q4;
+        for (int d = 0; d < MB; d++) {
+          if (16 * d + 4 * q4 < a.D) check_access("dk", dkp + 16 * d, 8, true);
+          if (16 * d + 4 * q4 < a.Dv) check_access("dv", dvp + 16 * d, 8, true);
+        }
+      }
+      Loader ld;
+      ld.init(tid);
+      const bool st_lse = (wave & 1) == 0;
+      const char* stb = st_lse ? (const char*)(a.lse + (int64_t)b * a.Tq * a.Hq + hkv) : (const char*)(a.delta + ((int64_t)b * a.Hq + hkv) * a.Tq);
+      const uint32_t st_row = st_lse ? (uint32_t)a.Hq * 4u : 4u;
+      int ld_st = 0;
+      for (int it = 0; it < plan.nqt; it++) {
+        const int f_q0 = (plan.qt0 + plan.nqt - 1 - it) * BM;
+        if (f_q0 < 0) fail("dkv_flat_kernel: query tile row %d", f_q0);
+        const uint32_t Qt = (uint32_t)(ld_st * 2 * BM * HD) * 2;
+        ctx("dkv_flat_kernel", (int)block, wave, lane, "query tile (Q, dO)");
+        for (int i = 0; i < Loader::N; i++) {
+          check_dma("q", a.q + b * a.sq.b + hkv * a.sq.h + (int64_t)f_q0 * a.sq.t, Loader::anchored_bytes(a.sq.t, f_q0, a.Tq),
+                    ld.lane_offset((int)a.sq.t * 2, a.D), Loader::rows_before(i) * (int)a.sq.t * 2, 16,
+                    Qt + (uint32_t)ld.lds_elems(i) * 2, lds_bytes, ld.pads(a.D));
+          check_dma("do", a.d_o + b * a.sdo.b + hkv * a.sdo.h + (int64_t)f_q0 * a.sdo.t, Loader::anchored_bytes(a.sdo.t, f_q0, a.Tq),
+                    ld.lane_offset((int)a.sdo.t * 2, a.Dv), Loader::rows_before(i) * (int)a.sdo.t * 2, 16,
+                    Qt + (uint32_t)(BM * HD + ld.lds_elems(i)) * 2, lds_bytes, ld.pads(a.Dv));
+        }
+        const int rows = imax(imin(a.Tq - f_q0, BM), 0);
+        if (rows == 0) fail("dkv_flat_kernel: empty query tile at row %d (Tq %d)", f_q0, a.Tq);
+        ctx("dkv_flat_kernel", (int)block, wave, lane, st_lse ? "query tile lse" : "query tile row sums");
+        check_dma(st_lse ? "lse" : "delta", stb + (int64_t)f_q0 * st_row, (uint32_t)(rows - 1) * st_row + 4u, lane * (int)st_row, 0, 4,
+                  stat_byte + (uint32_t)(ld_st * 2 * SP + (st_lse ? 0 : SP)) * 4, lds_bytes, false);
+        ld_st = (ld_st + 1) % NST;
+      }
+    }
+  }
+}
+
 // the partial sums of the row segments -> dk, dv
 template <int HD>
 void walk_reduce(const KArgs& a) {
@@ -785,7 +847,11 @@ void walk_all(const Case& c, const KArgs& a) {
     require_full("hand_p");
     require_full("hand_ds");
   }
-  walk_dkv<HD>(a);
+  if (takes_dkv_flat(a, HD, a.cu ? 1 : a.dkv_split)) {
+    if constexpr (HD == 64) walk_dkv_flat<HD>(a);
+  } else {
+    walk_dkv<HD>(a);
+  }
   if (a.dkv_split > 1 && a.has_seq) {
     require_full("part");
     walk_reduce<HD>(a);

@@ -854,9 +854,10 @@ def test_row_split_sequence_gradients(gpu_device, case):
     assert torch.equal(dq, got["dq"])
     check("dk", dk, ref["dk"], dtype, "unsplit")
     check("dv", dv, ref["dv"], dtype, "unsplit")
-    # the two summation orders agree to a rounding of the 16-bit result
+    # the two evaluations agree to a rounding or two of the 16-bit result (the unsplit launch of a short 64-wide case
+    # runs on the short-launch kernel, which rounds P once where the split kernel rounds it twice)
     for a, b_ in ((dk, got["dk"]), (dv, got["dv"])):
-        assert ((a.float() - b_.float()).abs() <= 2.0 ** -7 * b_.float().abs() + 1e-3).all()
+        assert ((a.float() - b_.float()).abs() <= 2.0 ** -6 * b_.float().abs() + 2e-3).all()
 
 
 def test_hip_graph_capture_and_replay(gpu_device):
