@@ -306,7 +306,7 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # what FETCH_SIZE / WRITE_SIZE (KiB per dispatch) read for a plain copy of known size (the depth reorganisation
 # kernel of the same runs): FETCH_SIZE counts half of the bytes read, WRITE_SIZE all bytes written
 PMC_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
-KERNEL_NAMES = ("fwd_kernel", "fwd_wide_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "dkv_reduce_kernel", "depth_cols_kernel",
+KERNEL_NAMES = ("fwd_kernel", "fwd_wide_kernel", "delta_kernel", "dq_kernel", "dkv_kernel", "dkv_flat_kernel", "dkv_reduce_kernel", "depth_cols_kernel",
                 "depth_token_handed_kernel", "depth_cols_handed_kernel", "chunk_depth_kernel", "reorg_kernel")
 
 
@@ -320,6 +320,15 @@ def depth_gradient_kernel(mode, D, G):
     if D <= 128:
         return "depth_token_handed_kernel" if G <= 4 else "depth_cols_handed_kernel"
     return "depth_cols_kernel"
+
+
+def sequence_dkv_kernel(B, T, Hkv, G, D, compute_units=256):
+    """Name of the launch that forms dk, dv of the sequence keys (moda_amd/csrc/geometry.h: takes_dkv_flat,
+    moda_amd/csrc/capi.hip: desired_dkv_split): short launches on the 64-wide tiles go to the kernel without the
+    role split."""
+    tiles = -(-T // 128) * B * Hkv
+    split = tiles < 512 and (-(-T * G // 64)) // 2 >= 16
+    return "dkv_flat_kernel" if D <= 64 and T * G <= 512 and tiles <= 3 * compute_units and not split else "dkv_kernel"
 
 
 def recorded_traffic(workload):
@@ -539,7 +548,8 @@ def main():
         mb = min_hbm_bytes(B, T, Hkv, G, D, L, mode)
         gbs = mb / (r["ms_step"] * 1e-3) / 1e9
         whole = sum(v["bytes"] for k, v in traffic.items() if k != "reorg_kernel") if traffic else None
-        launches = ["fwd_kernel", "dq_kernel"] + (["dkv_kernel"] if mode != "depth_only" else []) + ([depth_kernel] if depth_kernel else [])
+        launches = ["fwd_kernel", "dq_kernel"] + ([sequence_dkv_kernel(B, T, Hkv, G, D)] if mode != "depth_only" else []) \
+            + ([depth_kernel] if depth_kernel else [])
         roofline = {"bound": "hbm", "kernel": " + ".join(launches),
                     "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                     "algorithmic_bytes": mb, "traffic": whole,
