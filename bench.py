@@ -325,10 +325,10 @@ def depth_gradient_kernel(mode, D, G):
 def sequence_dkv_kernel(B, T, Hkv, G, D, compute_units=256):
     """Name of the launch that forms dk, dv of the sequence keys (moda_amd/csrc/geometry.h: takes_dkv_flat,
     moda_amd/csrc/capi.hip: desired_dkv_split): short launches on the 64-wide tiles go to the kernel without the
-    role split."""
+    role split when they are short or have at least three column tiles per compute unit."""
     tiles = -(-T // 128) * B * Hkv
     split = tiles < 512 and (-(-T * G // 64)) // 2 >= 16
-    return "dkv_flat_kernel" if D <= 64 and T * G <= 512 and tiles <= 3 * compute_units and not split else "dkv_kernel"
+    return "dkv_flat_kernel" if D <= 64 and not split and (T * G <= 512 or tiles >= 3 * compute_units) else "dkv_kernel"
 
 
 def recorded_traffic(workload):

@@ -1,5 +1,5 @@
-// Backward, key side, sequence keys of short fixed-length launches on the 64-wide tiles: the same products as
-// dkv_kernel (moda_v14.py:874-1248, fla/ops/attn/parallel.py:299-440) without the split into two roles.
+// Backward, key side, sequence keys of fixed-length launches on the 64-wide tiles: the same products as dkv_kernel
+// (moda_v14.py:874-1248, fla/ops/attn/parallel.py:299-440) without the split into two roles.
 //
 // A workgroup of FOUR waves owns 128 key columns of one (batch, kv head), a wave 32 of them with K AND V in
 // registers and BOTH accumulators, dK^T and dV^T; the query rows come by in tiles of 32 (one summation step of the
@@ -8,9 +8,10 @@
 //   dV^T += dO^T P, dK^T += Q^T dS.
 // P stays in fp32 until dS is formed (one rounding on the dK path) and nothing travels between waves.  With 26 KB of
 // LDS and no mailbox, three workgroups share a compute unit where dkv_kernel fits one: a launch of a few hundred
-// column tiles (a vision model's 197 tokens) runs in one round of workgroups instead of three.  On long sequences
-// the role split is the faster of the two by far (more matrix work per operand read), so this kernel only takes the
-// launches that fit the machine at once.
+// column tiles of a short sequence (a vision model's 197 tokens) runs in one round of workgroups instead of three,
+// and a launch with many column tiles keeps twelve waves per compute unit busy instead of eight.  A launch of few
+// tiles over a long sequence is bound by its heaviest tile, where the eight waves of dkv_kernel are faster; on the
+// 128-wide tiles this structure spills.  geometry.h: takes_dkv_flat says which launches come here.
 #include <type_traits>
 
 #include "geometry.h"

@@ -192,15 +192,17 @@ inline int64_t col_kernel_blocks(const KArgs& a, int HD, int BN, int nseg) {
   const int64_t n_dep_tiles = (a.L > 0 && a.chunk && !depth_by_chunks(a, HD)) ? ((int64_t)a.T * a.Lv + BN - 1) / BN : 0;
   return (n_seq_tiles * nseg + n_dep_tiles) * a.B * a.Hkv;
 }
-// Sequence dK/dV of short launches on the 64-wide tiles: dkv_flat_kernel (three workgroups per compute unit) takes
-// the launch when its column tiles -- sequence keys only, fixed length, kv head = query head, no row segments --
-// fit the machine in one round and see few query rows each (on a long sequence the role split of dkv_kernel does
-// more matrix work per operand read and wins: at 8192 rows by 18 %).
+// Sequence dK/dV on the 64-wide tiles: dkv_flat_kernel (three workgroups per compute unit, where dkv_kernel fits
+// one) takes a launch of sequence-key column tiles -- fixed length, kv head = query head, no row segments -- when the
+// tiles see few query rows each (the launch waits for memory, not for the matrix pipe) or when there are enough of
+// them to fill every compute unit's three places (measured: 18-35 % faster from 768 tiles up, at any sequence
+// length; 16-25 % slower at 512 tiles of 16 K rows, where the heaviest tile's trips set the time).
 constexpr int kDkvFlatMaxRows = 512;
 inline int64_t dkv_flat_blocks(const KArgs& a) { return a.has_seq ? (int64_t)((a.T + 127) / 128) * a.B * a.Hkv : 0; }
 inline bool takes_dkv_flat(const KArgs& a, int HD, int nseg) {
-  return HD == 64 && !a.cu && a.has_seq && a.hdiv == 1 && nseg == 1 && a.compute_units > 0 && a.Tq <= kDkvFlatMaxRows &&
-         col_kernel_blocks(a, HD, 128, 1) == dkv_flat_blocks(a) && dkv_flat_blocks(a) <= 3ll * a.compute_units;
+  return HD == 64 && !a.cu && a.has_seq && a.hdiv == 1 && nseg == 1 && a.compute_units > 0 &&
+         col_kernel_blocks(a, HD, 128, 1) == dkv_flat_blocks(a) &&
+         (a.Tq <= kDkvFlatMaxRows || dkv_flat_blocks(a) >= 3ll * a.compute_units);
 }
 inline int64_t delta_kernel_blocks(const KArgs& a, int rows_per_block) {
   return (int64_t)((a.Tq + rows_per_block - 1) / rows_per_block) * a.B * a.Hq;

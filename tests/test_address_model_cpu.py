@@ -101,6 +101,8 @@ FIXED = [
     (2, 90, 2, 128, 4, 3, "causal", 0, 0),
     (1, 50, 1, 64, 6, 5, "depth_only", 0, 4),
     (2, 1500, 1, 128, 3, 4, "causal", 0, 2),       # ... in the throughput launch shape, partially filled
+    # 64-wide tiles, more than 512 query rows, three sequence column tiles per compute unit: the four-wave dK/dV kernel
+    (12, 1024, 8, 64, 2, 2, "causal", 0, 0),
     # what the per-sequence route launches for the packed case above: one fixed-length problem per sequence
     (1, 70, 1, 192, 5, 4, "chunk_visible", 8, 0),
     (1, 200, 1, 192, 5, 4, "chunk_visible", 8, 0),

@@ -197,6 +197,10 @@ VARIANTS = [
     (2, 90, 2, 64, 4, 3, "causal", 0, torch.bfloat16),
     (1, 50, 1, 48, 6, 5, "depth_only", 0, torch.float16),
     (8, 520, 8, 64, 1, 4, "causal", 0, torch.bfloat16),
+    # 64-wide tiles with at least three sequence column tiles per compute unit and more than 512 query rows: the
+    # sequence dK/dV of these go to the four-wave kernel by the size of the grid, not by their length
+    (12, 1024, 8, 64, 2, 2, "causal", 0, torch.bfloat16),
+    (6, 1100, 16, 48, 0, 1, "noncausal", 0, torch.float16),
 ]
 
 
