@@ -1080,6 +1080,34 @@ def test_packed_batch_equals_separate_calls_bitwise(gpu_device):
             assert torch.equal(leaf[n].grad[:, a * mult[n]:b * mult[n]], one[key]), (i, n)
 
 
+def test_packed_batch_on_the_narrow_tiles_against_separate_calls(gpu_device):
+    """On the 64-wide tiles the separate (fixed-length, short) calls form dk, dv in the four-wave kernel, which rounds
+    the probabilities once, the packed launch in the role-split kernel, which rounds them twice: everything else is
+    bit-identical, dk and dv agree to that rounding."""
+    lengths, H, D, L, G = (197, 64, 1, 300), 2, 64, 4, 2
+    cu = _cu(lengths)
+    inp = to_dev(oracle.make_inputs(1, cu[-1], H, D, L, G, seed=41, dtype=torch.bfloat16, std=0.5), gpu_device)
+    from moda_amd import ops
+
+    m = MODE_ID["causal"]
+    packed = ops._packed(torch.tensor(cu, device=gpu_device), inp["q"], G)
+    o, lse = ops._raw_fwd(m, inp["q"], inp["k"], inp["v"], inp["kd"], inp["vd"], D ** -0.5, G, 0, packed=packed)
+    grads = ops._raw_bwd(m, inp["q"], inp["k"], inp["v"], inp["kd"], inp["vd"], o, lse, inp["do"], D ** -0.5, G, 0,
+                         packed=packed)
+    whole = dict(zip(("o", "lse", "dq", "dk", "dv", "dkd", "dvd"), (o, lse) + tuple(grads)))
+    mult = {"q": G, "k": 1, "v": 1, "kd": L, "vd": L}
+    for i in range(len(lengths)):
+        a, b = cu[i], cu[i + 1]
+        part = {n: inp[n][:, a * m:b * m] for n, m in mult.items()}
+        part["do"] = inp["do"][:, a * G:b * G]
+        one = run_hip(part, D ** -0.5, G, "causal", no_row_split=True)
+        for key, m in (("o", G), ("lse", G), ("dq", G), ("dkd", L), ("dvd", L)):
+            assert torch.equal(whole[key][:, a * m:b * m], one[key]), (i, key)
+        for key in ("dk", "dv"):
+            got, want = whole[key][:, a:b].float(), one[key].float()
+            assert ((got - want).abs() <= 2.0 ** -6 * want.abs() + 2e-3).all(), (i, key)
+
+
 def test_packed_plain_gqa_attention(gpu_device):
     import moda_amd
 
