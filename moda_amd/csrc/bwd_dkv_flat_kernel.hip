@@ -21,8 +21,9 @@
 
 namespace moda {
 
-template <typename T, int HD>
-__global__ __launch_bounds__(256, 3) void dkv_flat_kernel(const KArgs a) {
+// VARLEN: packed variable-length batch (a workgroup enters its sequence; column tiles past its end leave at once)
+template <typename T, int HD, bool VARLEN>
+__global__ __launch_bounds__(256, 3) void dkv_flat_kernel(const KArgs a_in) {
   constexpr int NB = 2, BM = 32, MBLK = BM / 16, BN = 4 * 16 * NB, KS = HD / 32, MB = HD / 16, NST = 3, DIST = 2;
   constexpr int SP = 64;  // floats per statistic and stage (one wave-wide load each)
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -31,11 +32,15 @@ __global__ __launch_bounds__(256, 3) void dkv_flat_kernel(const KArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int BHk = a.B * a.Hkv;
+  const int BHk = a_in.B * a_in.Hkv;
   const int bh = blockIdx.x % BHk;
   const int ct = blockIdx.x / BHk;
-  const int b = bh / a.Hkv, hkv = bh % a.Hkv;
-  const ColTilePlan plan = col_tile_plan(a, a, ct, BN, BM, false, 1);
+  int b = bh / a_in.Hkv;
+  const int hkv = bh % a_in.Hkv;
+  SeqArgs<VARLEN> seq(a_in, b);
+  const KArgs& a = seq.a;
+  const ColTilePlan plan = col_tile_plan(a_in, a, ct, BN, BM, VARLEN, 1);
+  if (VARLEN && !plan.active) return;  // a tile beyond this sequence of a variable-length batch
   int c[NB];
   bool valid[NB];
 #pragma unroll
@@ -76,7 +81,7 @@ __global__ __launch_bounds__(256, 3) void dkv_flat_kernel(const KArgs a) {
   // even waves fetch lse ([B, Tq, Hq]: one dword every Hq), odd waves minus delta ([B, Hq, Tq]: contiguous); the two
   // waves of a kind write the same values to the same place, which keeps every wave's load count per tile equal
   const bool st_lse = (wave & 1) == 0;
-  const char* stb = st_lse ? (const char*)(a.lse + (int64_t)b * a.Tq * a.Hq + hkv) : (const char*)(a.delta + ((int64_t)b * a.Hq + hkv) * a.Tq);
+  const char* stb = st_lse ? (const char*)(a.lse + (int64_t)b * a.Tq * a.Hq + hkv) : (const char*)(a.delta + ((int64_t)b * a.Hq + hkv) * (VARLEN ? a.delta_pitch : a.Tq));
   const uint32_t st_row = st_lse ? (uint32_t)a.Hq * 4u : 4u;
   const int voff_stat = lane * (int)st_row;
   int ld_st = 0;
@@ -214,22 +219,23 @@ __global__ __launch_bounds__(256, 3) void dkv_flat_kernel(const KArgs a) {
     }
 }
 
-template <typename T, int HD>
+template <typename T, int HD, bool VARLEN>
 hipError_t launch_dkv_flat_t(const KArgs& a, hipStream_t stream) {
   constexpr size_t smem = (size_t)3 * 2 * 32 * HD * sizeof(uint16_t) + 3 * 2 * 64 * sizeof(float);
   static LdsAttrState attr;
-  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_flat_kernel<T, HD>), smem);
+  const hipError_t ea = allow_dynamic_lds(attr, reinterpret_cast<const void*>(&dkv_flat_kernel<T, HD, VARLEN>), smem);
   if (ea != hipSuccess) return ea;
   const int64_t nblk = dkv_flat_blocks(a);
   if (nblk == 0) return hipSuccess;
   if (nblk >= (1ll << 31)) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((dkv_flat_kernel<T, HD>), dim3((unsigned)nblk), dim3(256), smem, stream, a);
+  hipLaunchKernelGGL((dkv_flat_kernel<T, HD, VARLEN>), dim3((unsigned)nblk), dim3(256), smem, stream, a);
   return hipGetLastError();
 }
 
 // dtype: 0 bf16, 1 fp16; 64-wide tiles only (the caller asks takes_dkv_flat first)
 hipError_t launch_dkv_flat(const KArgs& a, int dtype, hipStream_t stream) {
-  return dtype == 0 ? launch_dkv_flat_t<BF16, 64>(a, stream) : launch_dkv_flat_t<FP16, 64>(a, stream);
+  if (a.cu) return dtype == 0 ? launch_dkv_flat_t<BF16, 64, true>(a, stream) : launch_dkv_flat_t<FP16, 64, true>(a, stream);
+  return dtype == 0 ? launch_dkv_flat_t<BF16, 64, false>(a, stream) : launch_dkv_flat_t<FP16, 64, false>(a, stream);
 }
 
 }  // namespace moda

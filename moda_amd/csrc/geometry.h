@@ -193,14 +193,14 @@ inline int64_t col_kernel_blocks(const KArgs& a, int HD, int BN, int nseg) {
   return (n_seq_tiles * nseg + n_dep_tiles) * a.B * a.Hkv;
 }
 // Sequence dK/dV on the 64-wide tiles: dkv_flat_kernel (three workgroups per compute unit, where dkv_kernel fits
-// one) takes a launch of sequence-key column tiles -- fixed length, kv head = query head, no row segments -- when the
+// one) takes a launch of sequence-key column tiles -- kv head = query head, no row segments -- when the
 // tiles see few query rows each (the launch waits for memory, not for the matrix pipe) or when there are enough of
 // them to fill every compute unit's three places (measured: 18-35 % faster from 768 tiles up, at any sequence
 // length; 16-25 % slower at 512 tiles of 16 K rows, where the heaviest tile's trips set the time).
 constexpr int kDkvFlatMaxRows = 512;
 inline int64_t dkv_flat_blocks(const KArgs& a) { return a.has_seq ? (int64_t)((a.T + 127) / 128) * a.B * a.Hkv : 0; }
 inline bool takes_dkv_flat(const KArgs& a, int HD, int nseg) {
-  return HD == 64 && !a.cu && a.has_seq && a.hdiv == 1 && nseg == 1 && a.compute_units > 0 &&
+  return HD == 64 && a.has_seq && a.hdiv == 1 && nseg == 1 && a.compute_units > 0 &&
          col_kernel_blocks(a, HD, 128, 1) == dkv_flat_blocks(a) &&
          (a.Tq <= kDkvFlatMaxRows || dkv_flat_blocks(a) >= 3ll * a.compute_units);
 }

@@ -526,18 +526,25 @@ void walk_dkv(const KArgs& a_in) {
 
 // dkv_flat_kernel: four waves, a wave's 32 columns with K and V in registers, query tiles of 32 rows
 template <int HD>
-void walk_dkv_flat(const KArgs& a) {
+void walk_dkv_flat(const KArgs& a_in) {
   constexpr int NB = 2, BM = 32, BN = 4 * 16 * NB, KS = HD / 32, MB = HD / 16, NST = 3, SP = 64;
   const uint32_t lds_bytes = 3 * 2 * 32 * HD * 2 + 3 * 2 * 64 * 4;
   const uint32_t stat_byte = NST * 2 * BM * HD * 2;
-  const int BHk = a.B * a.Hkv;
-  const int64_t nblk = dkv_flat_blocks(a);
+  const bool varlen = a_in.cu != nullptr;
+  const int BHk = a_in.B * a_in.Hkv;
+  const int64_t nblk = dkv_flat_blocks(a_in);
   typedef AsyncTileLoader<HD, BM, 256> Loader;
   for (int64_t block = 0; block < nblk; block++) {
     const int bh = (int)(block % BHk), ct = (int)(block / BHk);
-    const int b = bh / a.Hkv, hkv = bh % a.Hkv;
-    const ColTilePlan plan = col_tile_plan(a, a, ct, BN, BM, false, 1);
-    if (!plan.active || plan.dep) fail("dkv_flat_kernel: column tile %d is not a sequence tile", ct);
+    int b = bh / a_in.Hkv;
+    const int hkv = bh % a_in.Hkv;
+    const KArgs a = seq_args(a_in, b);
+    const ColTilePlan plan = col_tile_plan(a_in, a, ct, BN, BM, varlen, 1);
+    if (!plan.active) {
+      if (!varlen) fail("dkv_flat_kernel: inactive column tile in a fixed-length launch");
+      continue;
+    }
+    if (plan.dep) fail("dkv_flat_kernel: column tile %d is not a sequence tile", ct);
     for (int tid = 0; tid < 256; tid++) {
       const int lane = tid & 63, n = lane & 15, q4 = lane >> 4, wave = tid >> 6;
       for (int nb = 0; nb < NB; nb++) {
@@ -559,7 +566,7 @@ void walk_dkv_flat(const KArgs& a) {
       Loader ld;
       ld.init(tid);
       const bool st_lse = (wave & 1) == 0;
-      const char* stb = st_lse ? (const char*)(a.lse + (int64_t)b * a.Tq * a.Hq + hkv) : (const char*)(a.delta + ((int64_t)b * a.Hq + hkv) * a.Tq);
+      const char* stb = st_lse ? (const char*)(a.lse + (int64_t)b * a.Tq * a.Hq + hkv) : (const char*)(a.delta + ((int64_t)b * a.Hq + hkv) * (varlen ? a.delta_pitch : a.Tq));
       const uint32_t st_row = st_lse ? (uint32_t)a.Hq * 4u : 4u;
       int ld_st = 0;
       for (int it = 0; it < plan.nqt; it++) {

@@ -1081,9 +1081,9 @@ def test_packed_batch_equals_separate_calls_bitwise(gpu_device):
 
 
 def test_packed_batch_on_the_narrow_tiles_against_separate_calls(gpu_device):
-    """On the 64-wide tiles the separate (fixed-length, short) calls form dk, dv in the four-wave kernel, which rounds
-    the probabilities once, the packed launch in the role-split kernel, which rounds them twice: everything else is
-    bit-identical, dk and dv agree to that rounding."""
+    """On the 64-wide tiles the separate (short) calls form dk, dv in the four-wave kernel, which rounds the
+    probabilities once; this packed launch (longest sequence above 512 query rows, few column tiles) in the
+    role-split kernel, which rounds them twice: everything else is bit-identical, dk and dv agree to that rounding."""
     lengths, H, D, L, G = (197, 64, 1, 300), 2, 64, 4, 2
     cu = _cu(lengths)
     inp = to_dev(oracle.make_inputs(1, cu[-1], H, D, L, G, seed=41, dtype=torch.bfloat16, std=0.5), gpu_device)
